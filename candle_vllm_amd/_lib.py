@@ -7,8 +7,26 @@ import os
 import re
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.environ.get("MI355_LIB_PATH") or os.path.join(_HERE, "libmi355vllm.so")   # env override: A/B builds
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "mi355_vllm.h")
+HYBRID_HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "mi355_hybrid.h")
+# The whole library, or ONE component of it built alone (`__graft_entry__.build_component`): a fresh checkout that only serves a
+# layer-list model compiles the block engine, the rope tables and the hybrid host layer, not the llama-family kernels.  A component
+# library exports (and this module binds) the component's symbols only; asking it for another component's entry point raises.
+COMPONENT_LIBS = {"hybrid": os.path.join(_HERE, "libmi355vllm_hybrid.so")}
+COMPONENT_PREFIXES = {"hybrid": ("mi355_be_", "mi355_pc_", "mi355_sched_", "mi355_hybrid_", "mi355_hyb_", "mi355_rope_", "mi355_last_error",
+                                 "mi355_clear_error", "mi355_effective_max_seq_len", "mi355_abi_struct_size",
+                                 "mi355_rms_norm", "mi355_layer_norm", "mi355_silu_mul", "mi355_add_f32", "mi355_cast",
+                                 "mi355_embedding_f32", "mi355_argmax_f32")}
+_FULL = os.path.join(_HERE, "libmi355vllm.so")
+COMPONENT = None
+LIB_PATH = os.environ.get("MI355_LIB_PATH")                                              # env override: A/B builds
+if not LIB_PATH:
+    LIB_PATH = _FULL
+    _want = os.environ.get("MI355_LIB_COMPONENT")
+    if _want and not os.path.exists(_FULL):
+        if _want not in COMPONENT_LIBS:
+            raise ImportError(f"MI355_LIB_COMPONENT={_want}: unknown component (known: {sorted(COMPONENT_LIBS)})")
+        COMPONENT, LIB_PATH = _want, COMPONENT_LIBS[_want]
 
 
 def declared_symbols(header_path=HEADER_PATH):
@@ -19,6 +37,10 @@ def declared_symbols(header_path=HEADER_PATH):
     return sorted(set(names))
 
 
+def _in_component(name):
+    return COMPONENT is None or name.startswith(COMPONENT_PREFIXES[COMPONENT])
+
+
 if not os.path.exists(LIB_PATH):
     raise ImportError(
         f"{LIB_PATH} not found: run `python __graft_entry__.py` (hipcc --offload-arch=gfx950) first; "
@@ -26,7 +48,7 @@ if not os.path.exists(LIB_PATH):
 
 lib = ctypes.CDLL(LIB_PATH, mode=ctypes.RTLD_GLOBAL)
 
-_missing = [s for s in declared_symbols() if not hasattr(lib, s)]
+_missing = [s for s in declared_symbols() + declared_symbols(HYBRID_HEADER_PATH) if _in_component(s) and not hasattr(lib, s)]
 if _missing:
     raise ImportError(f"{LIB_PATH} does not export: {_missing}")
 
@@ -61,6 +83,8 @@ class RopeScaling(ctypes.Structure):
 
 
 def _sig(name, restype, argtypes):
+    if not _in_component(name):
+        return None
     f = getattr(lib, name)
     f.restype = restype
     f.argtypes = argtypes
@@ -252,6 +276,7 @@ _sig("mi355_llama_set_rope_tables", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32])
 _sig("mi355_abi_struct_size", c_i64, [c_i32])
 _sig("mi355_rope_table_len", c_i32, [c_vp, c_i32, c_i32])
 _sig("mi355_rope_tables", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, ctypes.c_double, c_vp, c_i32, c_i32])
+_sig("mi355_rope_tables_f64", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, ctypes.c_double, c_vp, c_i32, c_i32])
 _sig("mi355_comm_create", c_vp, [c_vp, c_i32, c_i32])
 ALLREDUCE_FN = ctypes.CFUNCTYPE(ctypes.c_int, c_vp, c_vp, c_i64, c_i32, c_i64)
 ALLGATHER_FN = ctypes.CFUNCTYPE(ctypes.c_int, c_vp, c_vp, c_vp, c_i64, c_i32, c_i64)
@@ -308,8 +333,59 @@ _sig("mi355_gguf_tensor_shard_q8_0", ctypes.c_int64, [c_vp, c_i32, c_i32, c_i32,
 _sig("mi355_gguf_tensor_rows_padded", ctypes.c_int64, [c_vp, c_i32, ctypes.c_int64, ctypes.c_int64, c_vp, ctypes.c_int64])
 
 
+
+class HybridLayer(ctypes.Structure):
+    """mirror of `mi355_hybrid_layer` (include/mi355_hybrid.h)"""
+    _fields_ = [("mixer", c_i32),
+                ("a_heads", c_i32), ("a_kv_heads", c_i32), ("a_dim", c_i32), ("a_vdim", c_i32), ("a_window", c_i32),
+                ("a_rot_dims", c_i32), ("a_has_sink", c_i32), ("a_qk_norm", c_i32), ("a_scale", c_f32), ("a_out_scale", c_f32),
+                ("d_heads", c_i32), ("d_kv_heads", c_i32), ("d_dim", c_i32), ("d_vdim", c_i32), ("d_conv", c_i32),
+                ("d_decay_channels", c_i32), ("d_a_rank", c_i32), ("d_gate", c_i32), ("d_g_rank", c_i32), ("d_out_scale", c_f32),
+                ("g_width", c_i32), ("mlp_kind", c_i32), ("mlp_ff", c_i32), ("mlp_limit", c_f32), ("mlp_alpha", c_f32)]
+
+
+class HybridConfig(ctypes.Structure):
+    """mirror of `mi355_hybrid_config`"""
+    _fields_ = [("width", c_i32), ("vocab", c_i32), ("n_layers", c_i32), ("dtype", c_i32), ("block_size", c_i32),
+                ("state_slots", c_i32), ("norm_eps", c_f32), ("unit_eps", c_f32)]
+
+
+_sig("mi355_be_state_init", c_i32, [c_vp, c_i32])
+_sig("mi355_be_state_acquire", c_i32, [c_vp, c_i64])
+_sig("mi355_be_state_slot", c_i32, [c_vp, c_i64])
+_sig("mi355_be_state_free_slots", c_i32, [c_vp])
+_sig("mi355_be_seq_extend_prompt", c_i32, [c_vp, c_i64, c_vp, c_i32])
+_sig("mi355_hybrid_create", c_vp, [ctypes.POINTER(HybridConfig), ctypes.POINTER(HybridLayer)])
+_sig("mi355_hybrid_destroy", None, [c_vp])
+_sig("mi355_hybrid_in_proj_rows", c_i32, [ctypes.POINTER(HybridLayer), c_vp])
+_sig("mi355_hybrid_set_weight", ctypes.c_int, [c_vp, c_i32, c_i32, c_vp, c_i64])
+_sig("mi355_hybrid_set_weight_dev", ctypes.c_int, [c_vp, c_i32, c_i32, c_vp, c_i64, c_i64])
+_sig("mi355_hybrid_set_rope_tables", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32])
+_sig("mi355_hybrid_alloc_cache", ctypes.c_int, [c_vp, c_i32])
+_sig("mi355_hybrid_cache_bytes", c_i64, [c_vp, c_i32])
+_sig("mi355_hybrid_state_floats_per_slot", c_i64, [c_vp])
+_sig("mi355_hybrid_state_ptr", c_vp, [c_vp])
+_sig("mi355_hybrid_forward", ctypes.c_int, [c_vp] * 9 + [c_i32] * 5 + [c_vp, c_vp, c_i64])
+_sig("mi355_hyb_token_seq", ctypes.c_int, [c_vp, c_vp, c_i32, c_i64])
+_sig("mi355_hyb_bf16_to_f32", ctypes.c_int, [c_vp, c_vp, c_i64, c_i64])
+_sig("mi355_hyb_copy_f32", ctypes.c_int, [c_vp, c_vp, c_i64, c_i64])
+_sig("mi355_hyb_fill_f32", ctypes.c_int, [c_vp, c_f32, c_i64, c_i64])
+_sig("mi355_hyb_embed", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_i64])
+_sig("mi355_hyb_gather_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_linear", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_norm_add", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_attn_prepare", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_vp] * 6 + [c_i32] * 6 + [c_f32, c_i32, c_i64])
+_sig("mi355_hyb_window_attention", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 8 + [c_i32] * 9 + [c_f32, c_f32, c_i32, c_i64])
+_sig("mi355_hyb_conv_silu", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 4 + [c_i64])
+_sig("mi355_hyb_conv_state_update", ctypes.c_int, [c_vp, c_i64, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_delta_rule", ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp,
+                                              c_vp] + [c_i32] * 5 + [c_f32, c_i64])
+_sig("mi355_hyb_gated_norm", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_i64])
+_sig("mi355_hyb_mingru", ctypes.c_int, [c_vp, c_i32, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_clamped_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_f32, c_f32, c_i64])
+
 # the hand-written ctypes mirrors must have the layout the library was built with
-for _id, _cls in ((0, QmmDesc), (1, LlamaConfig), (2, DenseConfig), (3, RopeScaling)):
+for _id, _cls in ((0, QmmDesc), (1, LlamaConfig), (2, DenseConfig), (3, RopeScaling), (4, HybridConfig), (5, HybridLayer)):
     if lib.mi355_abi_struct_size(_id) != ctypes.sizeof(_cls):
         raise ImportError(f"{_cls.__name__}: ctypes mirror is {ctypes.sizeof(_cls)} bytes, the library expects "
                           f"{lib.mi355_abi_struct_size(_id)} (include/mi355_vllm.h changed?)")

@@ -53,6 +53,12 @@ class Sequence:
     def has_prefix_hash(self):
         return lib.mi355_be_seq_has_prefix_hash(self.engine.h, self.id) == 1
 
+    def extend_prompt(self, tokens):
+        """a prompt that arrives in portions: the tokens count as prompt, the next prompt step takes them"""
+        a, p, n = _tok(tokens)
+        if lib.mi355_be_seq_extend_prompt(self.engine.h, self.id, p, n) != 0:
+            raise ValueError("unknown sequence")
+
 
 class BlockEngine:
     """`BlockEngine::new(block_size, num_gpu_blocks, num_cpu_blocks, _, PrefixCacheConfig, false)`."""
@@ -204,6 +210,24 @@ class BlockEngine:
 
     def rollback_swap_in(self, gid):
         lib.mi355_be_rollback_swap_in(self.h, gid)
+
+    # -- recurrent-state slots (models whose layers carry state from token to token)
+    def state_init(self, n_slots):
+        if lib.mi355_be_state_init(self.h, int(n_slots)) != 0:
+            raise ValueError("state slots are set once, while no sequence holds one")
+
+    def state_acquire(self, seq):
+        """the sequence's slot; the lowest free one at the first call.  mi355_be_free_sequence gives it back with the blocks."""
+        r = lib.mi355_be_state_acquire(self.h, seq.id)
+        if r < 0:
+            raise RuntimeError("no free state slot" if r == -2 else "unknown sequence")
+        return r
+
+    def state_slot(self, seq):
+        return lib.mi355_be_state_slot(self.h, seq.id)
+
+    def state_free_slots(self):
+        return lib.mi355_be_state_free_slots(self.h)
 
     # -- input preparation (pipelines/inputs.rs)
     def prepare_decode(self, group):

@@ -17,6 +17,7 @@
 #include <cstdint>
 #include <cstring>
 #include <deque>
+#include <set>
 #include <unordered_map>
 #include <unordered_set>
 #include <vector>
@@ -217,6 +218,11 @@ struct Engine {
     std::unordered_map<int64_t, Seq> seqs;
     std::unordered_map<int64_t, Pending> pending_out, pending_in;
     int refuse_swap_out = 0, refuse_swap_in = 0;          // test hook (mi355_be_test_refuse_swaps): the next n swaps are refused up front
+    // recurrent-state slots of models whose layers carry state from token to token (mi355_be_state_*): one slot per live sequence,
+    // taken at its first step, given back with its blocks (mi355_be_free_sequence); lowest free slot first
+    std::set<int> state_free;
+    std::unordered_map<int64_t, int> state_of;
+    int state_slots = 0;
 
     int logical_blocks(const Seq& s) const { return (int)s.tokens.size() / block_size + 1; }     // sequence.rs:208-227
     int blocks_to_add_new_tok(const Seq& s) const { return (s.tokens.size() % block_size) == 0 ? 1 : 0; }
@@ -493,6 +499,39 @@ int32_t mi355_be_free_sequence(void* be, int64_t seq_id) {                      
     if (it == e->tables.end()) return -1;
     for (Blk b : it->second) e->release(b);
     e->tables.erase(it);
+    auto st = e->state_of.find(seq_id);
+    if (st != e->state_of.end()) { e->state_free.insert(st->second); e->state_of.erase(st); }
+    return 0;
+}
+/* ---- recurrent-state slots (no counterpart in the reference's block engine, which keeps the state of its hybrid models in the
+ * model runner): n slots in all; acquire = the sequence's slot, taking the lowest free one at the first call (-2: none free) */
+int32_t mi355_be_state_init(void* be, int32_t n_slots) {
+    Engine* e = E(be);
+    if (n_slots < 0 || !e->state_of.empty()) return -1;
+    e->state_free.clear();
+    for (int i = 0; i < n_slots; ++i) e->state_free.insert(i);
+    e->state_slots = n_slots;
+    return 0;
+}
+int32_t mi355_be_state_acquire(void* be, int64_t seq_id) {
+    Engine* e = E(be);
+    if (!find_seq(e, seq_id)) return -1;
+    auto it = e->state_of.find(seq_id);
+    if (it != e->state_of.end()) return it->second;
+    if (e->state_free.empty()) return -2;
+    const int slot = *e->state_free.begin();
+    e->state_free.erase(e->state_free.begin());
+    e->state_of[seq_id] = slot;
+    return slot;
+}
+int32_t mi355_be_state_slot(void* be, int64_t seq_id) { auto it = E(be)->state_of.find(seq_id); return it == E(be)->state_of.end() ? -1 : it->second; }
+int32_t mi355_be_state_free_slots(void* be) { return (int32_t)E(be)->state_free.size(); }
+/* a prompt that arrives in portions: the tokens are appended and count as prompt (the next prompt step takes them) */
+int32_t mi355_be_seq_extend_prompt(void* be, int64_t seq_id, const uint32_t* tokens, int32_t n) {
+    Seq* s = find_seq(E(be), seq_id);
+    if (!s || n < 0) return -1;
+    s->tokens.insert(s->tokens.end(), tokens, tokens + n);
+    s->prompt_len = (int)s->tokens.size();
     return 0;
 }
 int32_t mi355_be_cache_sequence(void* be, int64_t seq_id) {                                         // :594-646

@@ -1,0 +1,781 @@
+// Kernels of the layer-list ("hybrid") host layer (include/mi355_hybrid.h): sliding-window attention with a softmax sink over the
+// block engine's pages, the gated delta rule and the minGRU over the block engine's state slots, the short causal convolution in
+// front of the delta rule, and the f32-residual glue around them.  Numerics: residual stream, norms, scores, probabilities,
+// decays, gates of a recurrence and all recurrent state are f32; MI355_DTYPE_BF16 keeps matrices, K/V pages and the operands of
+// a matrix product in bf16 (matrix cores, f32 accumulation), MI355_DTYPE_F32 multiplies with f32 FMAs.
+// One step function serves prompts, portions of prompts and decoded tokens: a sequence brings cu_q[s+1] - cu_q[s] new tokens behind
+// ctx[s] - that many cached ones; a portion that starts at position 0 starts from zero state whatever its slot holds.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <math.h>
+
+#include "common.h"
+#include "../../include/mi355_hybrid.h"
+
+namespace {
+
+template <typename T> __device__ __forceinline__ float ld(const T* p, size_t i);
+template <> __device__ __forceinline__ float ld<float>(const float* p, size_t i) { return p[i]; }
+template <> __device__ __forceinline__ float ld<uint16_t>(const uint16_t* p, size_t i) { return bf16_to_f32(p[i]); }
+template <typename T> __device__ __forceinline__ void st(T* p, size_t i, float v);
+template <> __device__ __forceinline__ void st<float>(float* p, size_t i, float v) { p[i] = v; }
+template <> __device__ __forceinline__ void st<uint16_t>(uint16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
+    return v;
+}
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
+__device__ __forceinline__ float siluf_(float x) { return x / (1.f + expf(-x)); }
+__device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+
+// ------------------------------------------------------------------------------------------------------------ matrix products
+// 8 consecutive operands of a row as one MFMA fragment (bf16), zero beyond `kend`
+template <typename TA> __device__ __forceinline__ uint4 frag8(const TA* row, int k, int kend, bool vec_ok);
+template <> __device__ __forceinline__ uint4 frag8<uint16_t>(const uint16_t* row, int k, int kend, bool vec_ok) {
+    if (vec_ok && k + 8 <= kend) return *reinterpret_cast<const uint4*>(row + k);
+    uint16_t h[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) h[j] = (k + j < kend) ? row[k + j] : (uint16_t)0;
+    return uint4{(uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16),
+                 (uint32_t)h[4] | ((uint32_t)h[5] << 16), (uint32_t)h[6] | ((uint32_t)h[7] << 16)};
+}
+template <> __device__ __forceinline__ uint4 frag8<float>(const float* row, int k, int kend, bool vec_ok) {
+    float f[8];
+    if (vec_ok && k + 8 <= kend) {
+        const float4 a = *reinterpret_cast<const float4*>(row + k), b = *reinterpret_cast<const float4*>(row + k + 4);
+        f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+    } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = (k + j < kend) ? row[k + j] : 0.f;
+    }
+    return uint4{cvt_pk_bf16(f[0], f[1]), cvt_pk_bf16(f[2], f[3]), cvt_pk_bf16(f[4], f[5]), cvt_pk_bf16(f[6], f[7])};
+}
+__device__ __forceinline__ f32x4_t mfma_bf16(const uint4& a, const uint4& b, const f32x4_t& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+struct LinArgs {
+    float* out; int ldo;
+    const void* a; int lda;
+    const void* w; const float* bias;
+    int T, N, K;
+    int a_vec, w_vec;       // rows may be read 16 bytes at a time
+};
+
+// Prompt-sized products, bf16 weights.  A workgroup of four waves owns 64 output columns (16 weight rows per wave) and 16 MT tokens;
+// fragments go from global memory / L2 straight into registers: lane (m16, kg) holds operands 8 kg .. 8 kg + 7 of row m16 of a
+// 32-wide K step on both sides, the accumulator holds tokens 4 kg + v of column m16.
+template <typename TA, int MT> __global__ __launch_bounds__(256) void linear_bf16_tile_kernel(LinArgs p) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, kg = lane >> 4;
+    const int n = blockIdx.x * 64 + wave * 16 + m16;
+    const int t0 = blockIdx.y * (16 * MT);
+    const uint16_t* wrow = static_cast<const uint16_t*>(p.w) + (size_t)(n < p.N ? n : 0) * p.K;
+    const TA* arow[MT];
+    bool aok[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) {
+        const int t = t0 + i * 16 + m16;
+        aok[i] = t < p.T;
+        arow[i] = static_cast<const TA*>(p.a) + (size_t)(aok[i] ? t : 0) * p.lda;
+    }
+    f32x4_t acc[MT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i) acc[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const bool nok = n < p.N;
+    for (int k0 = 0; k0 < p.K; k0 += 32) {
+        const int k = k0 + 8 * kg;
+        const uint4 b = nok ? frag8<uint16_t>(wrow, k, p.K, p.w_vec) : uint4{0, 0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+            const uint4 a = aok[i] ? frag8<TA>(arow[i], k, p.K, p.a_vec) : uint4{0, 0, 0, 0};
+            acc[i] = mfma_bf16(a, b, acc[i]);
+        }
+    }
+    if (!nok) return;
+    const float bias = p.bias ? p.bias[n] : 0.f;
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int t = t0 + i * 16 + 4 * kg + v;
+            if (t < p.T) p.out[(size_t)t * p.ldo + n] = acc[i][v] + bias;
+        }
+}
+
+// Up to 16 tokens, bf16 weights: the product is a stream over the weights.  A workgroup owns 16 weight rows; its NW waves take the
+// 32-wide K steps in turn (UNR steps in flight per wave) and add their partial tiles through LDS.
+template <typename TA, int NW, int UNR> __global__ __launch_bounds__(64 * NW) void linear_bf16_stream_kernel(LinArgs p) {
+    __shared__ float part[NW][4][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, kg = lane >> 4;
+    const int n = blockIdx.x * 16 + m16;
+    const bool nok = n < p.N, aok = m16 < p.T;
+    const uint16_t* wrow = static_cast<const uint16_t*>(p.w) + (size_t)(nok ? n : 0) * p.K;
+    const TA* arow = static_cast<const TA*>(p.a) + (size_t)(aok ? m16 : 0) * p.lda;
+    f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int k0 = wave * 32 * UNR; k0 < p.K; k0 += NW * 32 * UNR) {
+        uint4 a[UNR], b[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) {
+            const int k = k0 + u * 32 + 8 * kg;
+            b[u] = (nok && k < p.K) ? frag8<uint16_t>(wrow, k, p.K, p.w_vec) : uint4{0, 0, 0, 0};
+            a[u] = (aok && k < p.K) ? frag8<TA>(arow, k, p.K, p.a_vec) : uint4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < UNR; ++u) acc = mfma_bf16(a[u], b[u], acc);
+    }
+#pragma unroll
+    for (int v = 0; v < 4; ++v) part[wave][v][lane] = acc[v];
+    __syncthreads();
+    if (wave == 0) {
+        const float bias = (p.bias && nok) ? p.bias[n] : 0.f;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) s += part[w][v][lane];
+            const int t = 4 * kg + v;
+            if (nok && t < p.T) p.out[(size_t)t * p.ldo + n] = s + bias;
+        }
+    }
+}
+
+// f32 weights and operands: plain FMAs in f32 (no reduced-precision matrix mode).  64 x 64 tile, 16-wide K steps through LDS,
+// every thread owns 4 tokens x 4 columns.
+__global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs p) {
+    __shared__ float As[16][68], Ws[16][68];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int n0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+    const float* A = static_cast<const float*>(p.a);
+    const float* W = static_cast<const float*>(p.w);
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < p.K; k0 += 16) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int idx = threadIdx.x + r * 256;            // 1024 elements of each 64 x 16 tile
+            const int row = idx >> 4, kk = idx & 15;
+            const int k = k0 + kk;
+            As[kk][row] = (t0 + row < p.T && k < p.K) ? A[(size_t)(t0 + row) * p.lda + k] : 0.f;
+            Ws[kk][row] = (n0 + row < p.N && k < p.K) ? W[(size_t)(n0 + row) * p.K + k] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; ++kk) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) { a[i] = As[kk][ty * 4 + i]; w[i] = Ws[kk][tx * 4 + i]; }
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int t = t0 + ty * 4 + i;
+        if (t >= p.T) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < p.N) p.out[(size_t)t * p.ldo + n] = acc[i][j] + (p.bias ? p.bias[n] : 0.f);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------ residual glue
+template <typename TW> __global__ void embed_kernel(float* x, uint16_t* xcopy, const TW* table, const uint32_t* ids, int width, int vocab) {
+    const int t = blockIdx.x;
+    const uint32_t id = ids[t] < (uint32_t)vocab ? ids[t] : 0u;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = ld<TW>(table, (size_t)id * width + i);
+        x[(size_t)t * width + i] = v;
+        if (xcopy) xcopy[(size_t)t * width + i] = f32_to_bf16(v);
+    }
+}
+
+__device__ __forceinline__ float block_sum(float v, float* red) {
+    v = wave_sum(v);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (int w = 0; w < nw; ++w) s += red[w];
+    return s;
+}
+
+// x += y / rms(y) * w  (the norm sits on the sublayer's OUTPUT), one workgroup per token
+__global__ __launch_bounds__(256) void norm_add_kernel(float* x, uint16_t* xcopy, const float* y, int ldy, const float* w, int width, float eps) {
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    const float* yr = y + (size_t)t * ldy;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) ss += yr[i] * yr[i];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = x[(size_t)t * width + i] + yr[i] * inv * w[i];
+        x[(size_t)t * width + i] = v;
+        if (xcopy) xcopy[(size_t)t * width + i] = f32_to_bf16(v);
+    }
+}
+
+// rows[r] of x -> RMS norm with weight -> out (dt) [n_rows, width]   (the model's last norm, on the wanted rows only)
+template <typename TO> __global__ __launch_bounds__(256) void gather_norm_kernel(TO* out, const float* x, const int32_t* rows, const float* w, int width, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    const float* xr = x + (size_t)rows[r] * width;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) ss += xr[i] * xr[i];
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) st<TO>(out, (size_t)r * width + i, xr[i] * inv * w[i]);
+}
+
+template <typename TO> __global__ void clamped_glu_kernel(TO* out, const float* gu, int64_t n, int ff, float limit, float alpha) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t t = i / ff; const int j = (int)(i - t * ff);
+    const float g = fminf(gu[t * 2 * ff + j], limit);
+    const float u = fminf(fmaxf(gu[t * 2 * ff + ff + j], -limit), limit);
+    st<TO>(out, (size_t)i, g * sigmoidf_(alpha * g) * (u + 1.f));
+}
+
+// ------------------------------------------------------------------------------------------------------------ attention
+struct PrepArgs {
+    void* q_out; void* k_pages; void* v_pages;
+    const float* proj; int ldp, q_off, k_off, v_off;
+    const float* qw; const float* kw; const float* cos_t; const float* sin_t;
+    const int64_t* positions; const int64_t* slots;
+    int H, G, d, vd, rot; float eps;
+};
+// one wave per (token, vector): query heads 0 .. H-1, key heads H .. H+G-1, value heads H+G .. H+2G-1
+template <typename TC> __global__ __launch_bounds__(64) void attn_prepare_kernel(PrepArgs p) {
+    extern __shared__ float vec[];
+    const int t = blockIdx.x, hv = blockIdx.y, lane = threadIdx.x;
+    const float* row = p.proj + (size_t)t * p.ldp;
+    const int64_t slot = p.slots[t];
+    if (hv >= p.H + p.G) {                                          // value head: a copy into the page
+        const int g = hv - p.H - p.G;
+        if (slot < 0) return;
+        TC* dst = static_cast<TC*>(p.v_pages) + ((size_t)slot * p.G + g) * p.vd;
+        for (int i = lane; i < p.vd; i += 64) st<TC>(dst, i, row[p.v_off + g * p.vd + i]);
+        return;
+    }
+    const bool is_q = hv < p.H;
+    const int h = is_q ? hv : hv - p.H;
+    const float* src = row + (is_q ? p.q_off : p.k_off) + h * p.d;
+    const float* w = is_q ? p.qw : p.kw;
+    float ss = 0.f;
+    for (int i = lane; i < p.d; i += 64) { const float v = src[i]; vec[i] = v; ss += v * v; }
+    ss = wave_sum(ss);
+    const float inv = w ? 1.f / sqrtf(ss / (float)p.d + p.eps) : 1.f;
+    __syncthreads();
+    for (int i = lane; i < p.d; i += 64) vec[i] = w ? vec[i] * inv * w[i] : vec[i];
+    __syncthreads();
+    TC* dst;
+    if (is_q) dst = static_cast<TC*>(p.q_out) + ((size_t)t * p.H + h) * p.d;
+    else { if (slot < 0) return; dst = static_cast<TC*>(p.k_pages) + ((size_t)slot * p.G + h) * p.d; }
+    const int half = p.rot / 2;
+    const int64_t pos = p.positions[t];
+    for (int i = lane; i < p.d; i += 64) {
+        float v = vec[i];
+        if (i < half) {
+            const float c = p.cos_t[pos * half + i], s = p.sin_t[pos * half + i];
+            v = vec[i] * c - vec[i + half] * s;
+        } else if (i < p.rot) {
+            const float c = p.cos_t[pos * half + i - half], s = p.sin_t[pos * half + i - half];
+            v = vec[i] * c + vec[i - half] * s;
+        }
+        st<TC>(dst, i, v);
+    }
+}
+
+struct AttnArgs {
+    void* out; int ldo, out_off;
+    const void* q; const void* k_pages; const void* v_pages;
+    const uint32_t* bt; const uint32_t* ctx; const uint32_t* cu_q; const int32_t* tok_seq; const float* sink;
+    int n_seqs, H, G, d, vd, bs, max_blocks, window; float scale, out_scale;
+};
+// One workgroup of NW waves per (new token, head).  Wave w takes the 64-key chunks w, w + NW, ... of the token's window: a lane
+// scores one key (q from LDS, the key row from its page), the wave keeps a running maximum / denominator / value sum (vd / 64
+// columns per lane), and the waves' partial results are merged through LDS.  The sink enters as a partial result with maximum
+// sink, denominator 1 and no value.
+template <typename TC, typename TO, int NW, int VPL> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
+    extern __shared__ float smem[];
+    float* qs = smem;                                   // [d]
+    float* pm = qs + p.d;                               // [NW] maxima, [NW] denominators, [NW][vd] sums
+    float* pl = pm + NW;
+    float* pacc = pl + NW;
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int s = p.tok_seq[t];
+    const int n_new = (int)(p.cu_q[s + 1] - p.cu_q[s]);
+    const int pos = (int)p.ctx[s] - n_new + (t - (int)p.cu_q[s]);
+    const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    const int g = h / (p.H / p.G);
+    const TC* q = static_cast<const TC*>(p.q) + ((size_t)t * p.H + h) * p.d;
+    for (int i = threadIdx.x; i < p.d; i += blockDim.x) qs[i] = ld<TC>(q, i);
+    __syncthreads();
+    const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
+    float m = -INFINITY, l = 0.f, acc[VPL];
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) acc[e] = 0.f;
+    for (int j0 = lo + wave * 64; j0 <= pos; j0 += NW * 64) {
+        const int j = j0 + lane;
+        float sc = -INFINITY;
+        unsigned page_row = 0;
+        if (j <= pos) {
+            page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
+            const TC* kr = static_cast<const TC*>(p.k_pages) + ((size_t)page_row * p.G + g) * p.d;
+            float dot = 0.f;
+            for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
+            sc = dot * p.scale;
+        }
+        const float mn = fmaxf(m, wave_max(sc));
+        const float pj = (j <= pos) ? expf(sc - mn) : 0.f;
+        const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
+        l = l * corr + wave_sum(pj);
+#pragma unroll
+        for (int e = 0; e < VPL; ++e) acc[e] *= corr;
+        m = mn;
+        const int cnt = min(64, pos - j0 + 1);
+        for (int jj = 0; jj < cnt; ++jj) {
+            const float pv = __shfl(pj, jj);
+            const size_t pr = (size_t)__shfl(page_row, jj);
+            const TC* vr = static_cast<const TC*>(p.v_pages) + (pr * p.G + g) * p.vd;
+#pragma unroll
+            for (int e = 0; e < VPL; ++e) { const int c = lane + 64 * e; if (c < p.vd) acc[e] = fmaf(pv, ld<TC>(vr, c), acc[e]); }
+        }
+    }
+    if (lane == 0) { pm[wave] = m; pl[wave] = l; }
+#pragma unroll
+    for (int e = 0; e < VPL; ++e) { const int c = lane + 64 * e; if (c < p.vd) pacc[wave * p.vd + c] = acc[e]; }
+    __syncthreads();
+    if (wave == 0) {
+        float M = p.sink ? p.sink[h] : -INFINITY;
+        for (int w = 0; w < NW; ++w) M = fmaxf(M, pm[w]);
+        float L = p.sink ? expf(p.sink[h] - M) : 0.f;
+        float o[VPL];
+#pragma unroll
+        for (int e = 0; e < VPL; ++e) o[e] = 0.f;
+        for (int w = 0; w < NW; ++w) {
+            if (pm[w] == -INFINITY) continue;
+            const float c = expf(pm[w] - M);
+            L += pl[w] * c;
+#pragma unroll
+            for (int e = 0; e < VPL; ++e) { const int col = lane + 64 * e; if (col < p.vd) o[e] += pacc[w * p.vd + col] * c; }
+        }
+        TO* out = static_cast<TO*>(p.out) + (size_t)t * p.ldo + p.out_off + (size_t)h * p.vd;
+#pragma unroll
+        for (int e = 0; e < VPL; ++e) { const int col = lane + 64 * e; if (col < p.vd) st<TO>(out, col, o[e] / L * p.out_scale); }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------ short convolution
+struct ConvArgs {
+    float* out; const float* proj; int ldp, off; const float* w; float* state; int64_t state_stride;
+    const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots; const int32_t* tok_seq; int C, taps, T;
+};
+__global__ void conv_silu_kernel(ConvArgs p) {
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)p.T * p.C) return;
+    const int t = (int)(idx / p.C), c = (int)(idx - (int64_t)t * p.C);
+    const int s = p.tok_seq[t];
+    const int cs = (int)p.cu_q[s];
+    const int start_pos = (int)p.ctx[s] - (int)(p.cu_q[s + 1] - p.cu_q[s]);
+    const float* stt = p.state + (size_t)p.slots[s] * p.state_stride + (size_t)c * (p.taps - 1);
+    float acc = 0.f;
+    for (int i = 0; i < p.taps; ++i) {
+        const int o = t - (p.taps - 1 - i);
+        float v;
+        if (o >= cs) v = p.proj[(size_t)o * p.ldp + p.off + c];
+        else {
+            const int back = cs - o;                                // 1 = the input just before the portion
+            v = (start_pos > 0 && start_pos - back >= 0) ? stt[p.taps - 1 - back] : 0.f;
+        }
+        acc = fmaf(p.w[(size_t)c * p.taps + i], v, acc);
+    }
+    p.out[idx] = siluf_(acc);
+}
+// state[j], j = 0 .. taps-2 (oldest first) <- the taps - 1 inputs that end with the portion's last token
+__global__ void conv_state_update_kernel(ConvArgs p, int n_seqs) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_seqs * p.C) return;
+    const int s = idx / p.C, c = idx - s * p.C;
+    const int cs = (int)p.cu_q[s], ce = (int)p.cu_q[s + 1], n = ce - cs;
+    if (n <= 0) return;
+    const int start_pos = (int)p.ctx[s] - n;
+    float* stt = p.state + (size_t)p.slots[s] * p.state_stride + (size_t)c * (p.taps - 1);
+    const int keep = p.taps - 1;
+    float nv[15];
+    for (int j = 0; j < keep; ++j) {
+        const int back = keep - j;                                   // 1 = the portion's last token
+        float v;
+        if (back <= n) v = p.proj[(size_t)(ce - back) * p.ldp + p.off + c];
+        else { const int b2 = back - n; v = (start_pos > 0 && start_pos - b2 >= 0) ? stt[keep - b2] : 0.f; }
+        nv[j] = v;
+    }
+    for (int j = 0; j < keep; ++j) stt[j] = nv[j];
+}
+
+// ------------------------------------------------------------------------------------------------------------ gated delta rule
+struct DeltaArgs {
+    float* o; float* state; int64_t state_stride;
+    const float* qkv; int ldq;
+    const float* proj; int ldp, b_off;
+    const float* decay_in; int ldd, decay_channels;
+    const float* a_log; const float* dt_bias;
+    const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots;
+    int H, G, d, vd; float unit_eps;
+};
+// One workgroup per (sequence, head); thread j owns column j of the state S [d, vd] in registers and walks the new tokens in order:
+//   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+// CH tokens at a time are staged in LDS: unit q (times d^-1/2), unit k, the decays and beta, computed by the whole workgroup.
+template <int D, int CH> __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs p) {
+    __shared__ float sq[CH][D], sk[CH][D], sg[CH][D];
+    __shared__ float sbeta[CH], sgh[CH];
+    const int s = blockIdx.x, h = blockIdx.y, nt = blockDim.x;
+    const int tid = blockIdx.z * nt + threadIdx.x;                  // the state column; a workgroup holds up to 256 of them
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = nt >> 6;
+    const int g = h / (p.H / p.G);
+    const int tb = (int)p.cu_q[s], te = (int)p.cu_q[s + 1];
+    if (te <= tb) return;
+    const int start_pos = (int)p.ctx[s] - (te - tb);
+    const int d = p.d, vd = p.vd;
+    const bool own = tid < vd;
+    float* stt = p.state + (size_t)p.slots[s] * p.state_stride + (size_t)h * d * vd;
+    float S[D];
+#pragma unroll
+    for (int i = 0; i < D; ++i) S[i] = (own && i < d && start_pos > 0) ? stt[(size_t)i * vd + tid] : 0.f;
+    const int q_col = g * d, k_col = p.G * d + g * d, v_col = 2 * p.G * d + h * vd;
+    const float a_rate = expf(p.a_log[h]);
+    const float q_scale = 1.f / sqrtf((float)d);
+    for (int t0 = tb; t0 < te; t0 += CH) {
+        const int cn = min(CH, te - t0);
+        __syncthreads();
+        // unit vectors: wave w normalises the q and k of tokens w, w + nw, ...
+        for (int c = wave; c < cn; c += nw) {
+            const float* row = p.qkv + (size_t)(t0 + c) * p.ldq;
+            float qq = 0.f, kk = 0.f;
+            for (int i = lane; i < d; i += 64) { const float a = row[q_col + i], b = row[k_col + i]; qq += a * a; kk += b * b; }
+            qq = wave_sum(qq); kk = wave_sum(kk);
+            const float qi = q_scale / sqrtf(qq + p.unit_eps), ki = 1.f / sqrtf(kk + p.unit_eps);
+            for (int i = lane; i < D; i += 64) {
+                sq[c][i] = i < d ? row[q_col + i] * qi : 0.f;
+                sk[c][i] = i < d ? row[k_col + i] * ki : 0.f;
+                if (p.decay_channels) {
+                    const int ch = h * d + i;
+                    sg[c][i] = i < d ? expf(-a_rate * softplusf_(p.decay_in[(size_t)(t0 + c) * p.ldd + ch] + p.dt_bias[ch])) : 1.f;
+                }
+            }
+            if (lane == 0) {
+                sbeta[c] = sigmoidf_(p.proj[(size_t)(t0 + c) * p.ldp + p.b_off + h]);
+                if (!p.decay_channels) sgh[c] = expf(-a_rate * softplusf_(p.decay_in[(size_t)(t0 + c) * p.ldd + h] + p.dt_bias[h]));
+            }
+        }
+        float vv[CH];
+#pragma unroll
+        for (int c = 0; c < CH; ++c) vv[c] = (own && c < cn) ? p.qkv[(size_t)(t0 + c) * p.ldq + v_col + tid] : 0.f;
+        __syncthreads();
+        if (own) {
+#pragma unroll 1
+            for (int c = 0; c < cn; ++c) {
+                float kv = 0.f;
+                if (p.decay_channels) {
+#pragma unroll
+                    for (int i = 0; i < D; ++i) { S[i] *= sg[c][i]; kv = fmaf(S[i], sk[c][i], kv); }
+                } else {
+                    const float gh = sgh[c];
+#pragma unroll
+                    for (int i = 0; i < D; ++i) { S[i] *= gh; kv = fmaf(S[i], sk[c][i], kv); }
+                }
+                const float u = sbeta[c] * (vv[c] - kv);
+                float o = 0.f;
+#pragma unroll
+                for (int i = 0; i < D; ++i) { S[i] = fmaf(sk[c][i], u, S[i]); o = fmaf(S[i], sq[c][i], o); }
+                p.o[((size_t)(t0 + c) * p.H + h) * vd + tid] = o;
+            }
+        }
+    }
+    if (own)
+#pragma unroll
+        for (int i = 0; i < D; ++i) if (i < d) stt[(size_t)i * vd + tid] = S[i];
+}
+
+// out = o / rms(o) * w * gate * out_scale, one wave per (token, head)
+template <typename TO> __global__ __launch_bounds__(64) void gated_norm_kernel(TO* out, int ldo, int out_off, const float* o, const float* w,
+                                                                              const float* gate_in, int ldg, int gate, int H, int vd,
+                                                                              float eps, float out_scale) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* orow = o + ((size_t)t * H + h) * vd;
+    float ss = 0.f;
+    for (int i = lane; i < vd; i += 64) ss += orow[i] * orow[i];
+    ss = wave_sum(ss);
+    const float inv = 1.f / sqrtf(ss / (float)vd + eps);
+    for (int i = lane; i < vd; i += 64) {
+        const float gi = gate_in[(size_t)t * ldg + h * vd + i];
+        const float gt = gate == MI355_HYB_GATE_SILU ? siluf_(gi) : sigmoidf_(gi);
+        st<TO>(out, (size_t)t * ldo + out_off + h * vd + i, orow[i] * inv * w[i] * gt * out_scale);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------ minGRU
+struct GruArgs {
+    void* out; float* state; int64_t state_stride; const float* proj; int ldp, z_off, x_off, g_off;
+    const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots; int width;
+};
+// thread = (sequence, channel); the gates read only the current token, so their loads run UNR tokens ahead of the recurrence
+template <typename TO, int UNR> __global__ __launch_bounds__(64) void mingru_kernel(GruArgs p) {
+    const int s = blockIdx.y, c = blockIdx.x * 64 + threadIdx.x;
+    if (c >= p.width) return;
+    const int tb = (int)p.cu_q[s], te = (int)p.cu_q[s + 1];
+    if (te <= tb) return;
+    const int start_pos = (int)p.ctx[s] - (te - tb);
+    float* stt = p.state + (size_t)p.slots[s] * p.state_stride;
+    float S = start_pos > 0 ? stt[c] : 0.f;
+    for (int t0 = tb; t0 < te; t0 += UNR) {
+        float z[UNR], u[UNR], gg[UNR];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            const int t = min(t0 + k, te - 1);
+            const float* row = p.proj + (size_t)t * p.ldp;
+            z[k] = row[p.z_off + c]; u[k] = row[p.x_off + c]; gg[k] = row[p.g_off + c];
+        }
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            if (t0 + k >= te) break;
+            const float zz = sigmoidf_(z[k]);
+            const float cand = u[k] >= 0.f ? u[k] + 0.5f : sigmoidf_(u[k]);
+            S = (1.f - zz) * S + zz * cand;
+            st<TO>(static_cast<TO*>(p.out), (size_t)(t0 + k) * p.width + c, S * siluf_(gg[k]));
+        }
+    }
+    stt[c] = S;
+}
+
+__global__ void token_seq_kernel(int32_t* tok_seq, const uint32_t* cu_q, int n_seqs) {
+    const int s = blockIdx.x;
+    for (int t = (int)cu_q[s] + threadIdx.x; t < (int)cu_q[s + 1]; t += blockDim.x) tok_seq[t] = s;
+}
+__global__ void bf16_to_f32_kernel(float* out, const uint16_t* in, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = bf16_to_f32(in[i]);
+}
+__global__ void copy_f32_kernel(float* out, const float* in, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = in[i];
+}
+__global__ void fill_f32_kernel(float* out, float v, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = v;
+}
+
+#define LAUNCH_OK() do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)
+inline bool is_dt(int dt) { return dt == MI355_DTYPE_F32 || dt == MI355_DTYPE_BF16; }
+
+}  // namespace
+
+extern "C" {
+
+// sequence index of every token row (device helper of the host layer and of the standalone entry points)
+int mi355_hyb_token_seq(int32_t* tok_seq, const uint32_t* cu_seqlens_q, int32_t num_seqs, int64_t stream) {
+    if (num_seqs <= 0) return 0;
+    token_seq_kernel<<<num_seqs, 64, 0, to_stream(stream)>>>(tok_seq, cu_seqlens_q, num_seqs);
+    LAUNCH_OK(); return 0;
+}
+int mi355_hyb_bf16_to_f32(float* out, const uint16_t* in, int64_t n, int64_t stream) {
+    if (n <= 0) return 0;
+    bf16_to_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(out, in, n);
+    LAUNCH_OK(); return 0;
+}
+int mi355_hyb_copy_f32(float* out, const float* in, int64_t n, int64_t stream) {
+    if (n <= 0) return 0;
+    copy_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(out, in, n);
+    LAUNCH_OK(); return 0;
+}
+int mi355_hyb_fill_f32(float* out, float v, int64_t n, int64_t stream) {
+    if (n <= 0) return 0;
+    fill_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(out, v, n);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_linear(float* out, int32_t ldo, const void* a, int32_t a_dtype, int32_t lda, const void* w, const float* bias,
+                     int32_t T, int32_t n, int32_t k, int32_t dtype, int64_t stream) {
+    if (!out || !a || !w || T < 0 || n <= 0 || k <= 0 || ldo < n || lda < k || !is_dt(dtype) || !is_dt(a_dtype)) return -1;
+    if (T == 0) return 0;
+    LinArgs p{out, ldo, a, lda, w, bias, T, n, k, 0, 0};
+    hipStream_t st_ = to_stream(stream);
+    if (dtype == MI355_DTYPE_F32) {
+        if (a_dtype != MI355_DTYPE_F32) return -1;
+        linear_f32_kernel<<<dim3((n + 63) / 64, (T + 63) / 64), 256, 0, st_>>>(p);
+        LAUNCH_OK(); return 0;
+    }
+    const int a_bytes = a_dtype == MI355_DTYPE_F32 ? 4 : 2;
+    p.w_vec = (k % 8 == 0) && ((uintptr_t)w % 16 == 0);
+    p.a_vec = ((size_t)lda * a_bytes % 16 == 0) && ((uintptr_t)a % 16 == 0);
+    const bool af = a_dtype == MI355_DTYPE_F32;
+    if (T <= 16) {
+        const dim3 grid((n + 15) / 16);
+        if (k >= 2048) { if (af) linear_bf16_stream_kernel<float, 4, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 4, 4><<<grid, 256, 0, st_>>>(p); }
+        else { if (af) linear_bf16_stream_kernel<float, 2, 2><<<grid, 128, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 2, 2><<<grid, 128, 0, st_>>>(p); }
+    } else if (T <= 32) {
+        const dim3 grid((n + 63) / 64, (T + 31) / 32);
+        if (af) linear_bf16_tile_kernel<float, 2><<<grid, 256, 0, st_>>>(p); else linear_bf16_tile_kernel<uint16_t, 2><<<grid, 256, 0, st_>>>(p);
+    } else {
+        const dim3 grid((n + 63) / 64, (T + 63) / 64);
+        if (af) linear_bf16_tile_kernel<float, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_tile_kernel<uint16_t, 4><<<grid, 256, 0, st_>>>(p);
+    }
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_embed(float* x, void* xcopy, const void* table, const uint32_t* ids, int32_t T, int32_t width, int32_t vocab, int32_t dtype,
+                    int64_t stream) {
+    if (!x || !table || !ids || !is_dt(dtype) || width <= 0) return -1;
+    if (T <= 0) return 0;
+    if (dtype == MI355_DTYPE_F32) embed_kernel<float><<<T, 256, 0, to_stream(stream)>>>(x, (uint16_t*)xcopy, (const float*)table, ids, width, vocab);
+    else embed_kernel<uint16_t><<<T, 256, 0, to_stream(stream)>>>(x, (uint16_t*)xcopy, (const uint16_t*)table, ids, width, vocab);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_norm_add(float* x, void* xcopy, const float* y, int32_t ldy, const float* w, int32_t T, int32_t width, float eps,
+                       int64_t stream) {
+    if (!x || !y || !w || width <= 0 || ldy < width) return -1;
+    if (T <= 0) return 0;
+    norm_add_kernel<<<T, 256, 0, to_stream(stream)>>>(x, (uint16_t*)xcopy, y, ldy, w, width, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_gather_norm(void* out, int32_t out_dtype, const float* x, const int32_t* rows, const float* w, int32_t n_rows, int32_t width,
+                          float eps, int64_t stream) {
+    if (!out || !x || !rows || !w || !is_dt(out_dtype)) return -1;
+    if (n_rows <= 0) return 0;
+    if (out_dtype == MI355_DTYPE_F32) gather_norm_kernel<float><<<n_rows, 256, 0, to_stream(stream)>>>((float*)out, x, rows, w, width, eps);
+    else gather_norm_kernel<uint16_t><<<n_rows, 256, 0, to_stream(stream)>>>((uint16_t*)out, x, rows, w, width, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_clamped_glu(void* out, int32_t out_dtype, const float* gu, int32_t T, int32_t ff, float limit, float alpha, int64_t stream) {
+    if (!out || !gu || ff <= 0 || !is_dt(out_dtype)) return -1;
+    const int64_t n = (int64_t)T * ff;
+    if (n <= 0) return 0;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (out_dtype == MI355_DTYPE_F32) clamped_glu_kernel<float><<<grid, 256, 0, to_stream(stream)>>>((float*)out, gu, n, ff, limit, alpha);
+    else clamped_glu_kernel<uint16_t><<<grid, 256, 0, to_stream(stream)>>>((uint16_t*)out, gu, n, ff, limit, alpha);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_attn_prepare(void* q_out, void* k_pages, void* v_pages, const float* proj, int32_t ldp, int32_t q_off, int32_t k_off,
+                           int32_t v_off, const float* q_norm_w, const float* k_norm_w, const float* cos_t, const float* sin_t,
+                           const int64_t* positions, const int64_t* slot_mapping, int32_t T, int32_t heads, int32_t kv_heads,
+                           int32_t dim, int32_t vdim, int32_t rot_dims, float eps, int32_t dtype, int64_t stream) {
+    if (!q_out || !k_pages || !v_pages || !proj || !positions || !slot_mapping || !is_dt(dtype)) return -1;
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1)) return -1;
+    if (rot_dims > 0 && (!cos_t || !sin_t)) return -1;
+    if (T <= 0) return 0;
+    PrepArgs p{q_out, k_pages, v_pages, proj, ldp, q_off, k_off, v_off, q_norm_w, k_norm_w, cos_t, sin_t, positions, slot_mapping,
+               heads, kv_heads, dim, vdim, rot_dims, eps};
+    const dim3 grid(T, heads + 2 * kv_heads);
+    if (dtype == MI355_DTYPE_F32) attn_prepare_kernel<float><<<grid, 64, dim * sizeof(float), to_stream(stream)>>>(p);
+    else attn_prepare_kernel<uint16_t><<<grid, 64, dim * sizeof(float), to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                                   const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                                   const uint32_t* cu_seqlens_q, const int32_t* tok_seq, const float* sink, int32_t num_seqs,
+                                   int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
+                                   int32_t max_blocks, int32_t window, float scale, float out_scale, int32_t dtype, int64_t stream) {
+    if (!out || !q || !k_pages || !v_pages || !block_tables || !context_lens || !cu_seqlens_q || !tok_seq) return -1;
+    if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || vdim > 512) return -1;
+    if (block_size <= 0 || max_blocks <= 0 || window < 0) return -1;
+    if (T <= 0) return 0;
+    AttnArgs p{out, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq, sink,
+               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale};
+    constexpr int NW = 4;
+    const size_t lds = (size_t)(dim + 2 * NW + NW * vdim) * sizeof(float);
+    const dim3 grid(T, heads);
+    hipStream_t s_ = to_stream(stream);
+    const bool f = dtype == MI355_DTYPE_F32, of = out_dtype == MI355_DTYPE_F32;
+#define WA(TC, TO, VPL) window_attention_kernel<TC, TO, NW, VPL><<<grid, 64 * NW, lds, s_>>>(p)
+#define WA_V(TC, TO) do { if (vdim <= 64) WA(TC, TO, 1); else if (vdim <= 128) WA(TC, TO, 2); else if (vdim <= 256) WA(TC, TO, 4); else WA(TC, TO, 8); } while (0)
+    if (f && of) WA_V(float, float); else if (f) WA_V(float, uint16_t); else if (of) WA_V(uint16_t, float); else WA_V(uint16_t, uint16_t);
+#undef WA_V
+#undef WA
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_conv_silu(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* conv_state,
+                            int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                            const int32_t* state_slots, const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t channels,
+                            int32_t taps, int64_t stream) {
+    if (!out || !proj || !w || !conv_state || !context_lens || !cu_seqlens_q || !state_slots || !tok_seq) return -1;
+    if (channels <= 0 || taps < 1 || taps > 16) return -1;
+    if (T <= 0) return 0;
+    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T};
+    const int64_t n = (int64_t)T * channels;
+    conv_silu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_conv_state_update(float* conv_state, int64_t state_stride, const float* proj, int32_t ldp, int32_t off,
+                                const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                                int32_t num_seqs, int32_t channels, int32_t taps, int64_t stream) {
+    if (!conv_state || !proj || !context_lens || !cu_seqlens_q || !state_slots || channels <= 0 || taps < 1 || taps > 16) return -1;
+    if (num_seqs <= 0 || taps == 1) return 0;
+    ConvArgs p{nullptr, proj, ldp, off, nullptr, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, nullptr, channels, taps, 0};
+    const int n = num_seqs * channels;
+    conv_state_update_kernel<<<(n + 255) / 256, 256, 0, to_stream(stream)>>>(p, num_seqs);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_delta_rule(float* o, float* state, int64_t state_stride, const float* qkv, int32_t ldq, const float* proj, int32_t ldp,
+                         int32_t b_off, const float* decay_in, int32_t ldd, int32_t decay_channels, const float* a_log,
+                         const float* dt_bias, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                         int32_t num_seqs, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float unit_eps, int64_t stream) {
+    if (!o || !state || !qkv || !proj || !decay_in || !a_log || !dt_bias || !context_lens || !cu_seqlens_q || !state_slots) return -1;
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > 256 || vdim <= 0) return -1;
+    if (num_seqs <= 0) return 0;
+    DeltaArgs p{o, state, state_stride, qkv, ldq, proj, ldp, b_off, decay_in, ldd, decay_channels, a_log, dt_bias,
+                context_lens, cu_seqlens_q, state_slots, heads, kv_heads, dim, vdim, unit_eps};
+    const int threads = vdim >= 256 ? 256 : ((vdim + 63) / 64) * 64;
+    const dim3 grid(num_seqs, heads, (vdim + threads - 1) / threads);
+    hipStream_t s_ = to_stream(stream);
+    if (dim <= 16) delta_rule_kernel<16, 8><<<grid, threads, 0, s_>>>(p);
+    else if (dim <= 32) delta_rule_kernel<32, 8><<<grid, threads, 0, s_>>>(p);
+    else if (dim <= 64) delta_rule_kernel<64, 8><<<grid, threads, 0, s_>>>(p);
+    else if (dim <= 128) delta_rule_kernel<128, 8><<<grid, threads, 0, s_>>>(p);
+    else delta_rule_kernel<256, 4><<<grid, threads, 0, s_>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_gated_norm(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const float* o, const float* w,
+                         const float* gate_in, int32_t ldg, int32_t gate, int32_t T, int32_t heads, int32_t vdim, float eps,
+                         float out_scale, int64_t stream) {
+    if (!out || !o || !w || !gate_in || !is_dt(out_dtype) || heads <= 0 || vdim <= 0) return -1;
+    if (T <= 0) return 0;
+    const dim3 grid(T, heads);
+    if (out_dtype == MI355_DTYPE_F32) gated_norm_kernel<float><<<grid, 64, 0, to_stream(stream)>>>((float*)out, ldo, out_off, o, w, gate_in, ldg, gate, heads, vdim, eps, out_scale);
+    else gated_norm_kernel<uint16_t><<<grid, 64, 0, to_stream(stream)>>>((uint16_t*)out, ldo, out_off, o, w, gate_in, ldg, gate, heads, vdim, eps, out_scale);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_mingru(void* out, int32_t out_dtype, float* state, int64_t state_stride, const float* proj, int32_t ldp, int32_t z_off,
+                     int32_t x_off, int32_t g_off, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                     const int32_t* state_slots, int32_t num_seqs, int32_t width, int64_t stream) {
+    if (!out || !state || !proj || !context_lens || !cu_seqlens_q || !state_slots || !is_dt(out_dtype) || width <= 0) return -1;
+    if (num_seqs <= 0) return 0;
+    GruArgs p{out, state, state_stride, proj, ldp, z_off, x_off, g_off, context_lens, cu_seqlens_q, state_slots, width};
+    const dim3 grid((width + 63) / 64, num_seqs);
+    if (out_dtype == MI355_DTYPE_F32) mingru_kernel<float, 8><<<grid, 64, 0, to_stream(stream)>>>(p);
+    else mingru_kernel<uint16_t, 8><<<grid, 64, 0, to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+}  // extern "C"

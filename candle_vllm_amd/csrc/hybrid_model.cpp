@@ -1,0 +1,422 @@
+// Host layer of the layer-list ("hybrid") models (include/mi355_hybrid.h): a model is a list of layers, each with one token mixer
+// (sliding-window attention with a sink, gated delta rule, minGRU, or attention and delta rule side by side) and an optional
+// feed-forward; x <- x + norm(mixer(x)), x <- x + norm(ff(x)), the sublayers read x itself.  Like the llama-family host layers
+// (host_model.cpp, dense_model.cpp) it owns the weights, the K/V pages and the activation buffers and enqueues one step on a
+// stream; unlike them it owns a pool of recurrent state (one slot per live sequence, handed out by the block engine) and runs
+// prompts, portions of prompts and decoded tokens through the same launches.
+// Kernels: hybrid_kernels.hip.  Every projection that reads a mixer's input is one matrix (rows concatenated at load time), the
+// output projections of a parallel mixer are one matrix along k (the branch scales are applied to the operands, not the weights).
+#include <hip/hip_runtime.h>
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <vector>
+
+#include "../../include/mi355_hybrid.h"
+
+#define MI355_DTYPE_F32 0
+#define MI355_DTYPE_BF16 2
+
+extern "C" {
+int mi355_hyb_token_seq(int32_t*, const uint32_t*, int32_t, int64_t);
+int mi355_hyb_bf16_to_f32(float*, const uint16_t*, int64_t, int64_t);
+int mi355_hyb_fill_f32(float*, float, int64_t, int64_t);
+int mi355_hyb_embed(float*, void*, const void*, const uint32_t*, int32_t, int32_t, int32_t, int32_t, int64_t);
+int mi355_hyb_gather_norm(void*, int32_t, const float*, const int32_t*, const float*, int32_t, int32_t, float, int64_t);
+}
+
+namespace {
+
+#define HCHECK(expr) do { const int rc_ = (expr); if (rc_ != 0) return rc_; } while (0)
+#define HHIP(expr) do { const hipError_t e_ = (expr); if (e_ != hipSuccess) return (int)e_; } while (0)
+
+enum { P_AQ = 0, P_AK, P_AV, P_DQ, P_DK, P_DV, P_B, P_A, P_G, P_COUNT };   // parts of the input projection (minGRU: z, x, g in 0..2)
+
+struct Weight { void* p = nullptr; int64_t n = 0; };
+
+struct HLayer {
+    mi355_hybrid_layer c{};
+    Weight w[MI355_HW_COUNT];
+    int32_t off[P_COUNT];
+    int32_t in_rows = 0, out_k = 0;
+    float *cos_t = nullptr, *sin_t = nullptr; int n_pos = 0;
+    void *k_pages = nullptr, *v_pages = nullptr;
+    int64_t conv_off = 0, state_off = 0;          // floats from the start of a slot
+    bool has_attn() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION; }
+    bool has_delta() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA; }
+    int conv_channels() const { return 2 * c.d_kv_heads * c.d_dim + c.d_heads * c.d_vdim; }
+};
+
+struct HModel {
+    mi355_hybrid_config cfg{};
+    std::vector<HLayer> layers;
+    Weight embed, final_norm, head;
+    int64_t slot_floats = 0;
+    float* state = nullptr;
+    int num_blocks = 0;
+    // activations (grow-only)
+    int cap_t = 0, cap_out = 0;
+    float *x = nullptr, *proj = nullptr, *aux1 = nullptr, *aux2 = nullptr, *conv = nullptr, *o = nullptr, *y = nullptr, *gu = nullptr;
+    void *xcopy = nullptr, *q = nullptr, *mix = nullptr, *act = nullptr, *xn = nullptr;
+    int32_t* tok_seq = nullptr;
+    int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0;
+    bool bf16() const { return cfg.dtype == MI355_DTYPE_BF16; }
+    size_t esize() const { return bf16() ? 2 : 4; }
+};
+
+int in_proj_parts(const mi355_hybrid_layer& c, int32_t* off) {
+    for (int i = 0; i < P_COUNT; ++i) off[i] = -1;
+    int r = 0;
+    if (c.mixer == MI355_HYB_MIX_MINGRU) {
+        off[0] = 0; off[1] = c.g_width; off[2] = 2 * c.g_width;
+        return 3 * c.g_width;
+    }
+    if (c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION) {
+        off[P_AQ] = r; r += c.a_heads * c.a_dim;
+        off[P_AK] = r; r += c.a_kv_heads * c.a_dim;
+        off[P_AV] = r; r += c.a_kv_heads * c.a_vdim;
+    }
+    if (c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA) {
+        off[P_DQ] = r; r += c.d_kv_heads * c.d_dim;
+        off[P_DK] = r; r += c.d_kv_heads * c.d_dim;
+        off[P_DV] = r; r += c.d_heads * c.d_vdim;
+        off[P_B] = r; r += c.d_heads;
+        off[P_A] = r; r += c.d_decay_channels ? c.d_a_rank : c.d_heads;
+        off[P_G] = r; r += c.d_gate == MI355_HYB_GATE_SIGMOID_LR ? c.d_g_rank : c.d_heads * c.d_vdim;
+    }
+    return r;
+}
+
+bool layer_ok(const mi355_hybrid_layer& c) {
+    const bool attn = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION;
+    const bool delta = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA;
+    if (c.mixer < 0 || c.mixer > MI355_HYB_MIX_ATTENTION) return false;
+    if (attn) {
+        if (c.a_heads <= 0 || c.a_kv_heads <= 0 || c.a_heads % c.a_kv_heads || c.a_dim <= 0 || c.a_vdim <= 0 || c.a_vdim > 512) return false;
+        if (c.a_window < 0 || c.a_rot_dims < 0 || c.a_rot_dims > c.a_dim || (c.a_rot_dims & 1)) return false;
+    }
+    if (delta) {
+        if (c.d_heads <= 0 || c.d_kv_heads <= 0 || c.d_heads % c.d_kv_heads || c.d_dim <= 0 || c.d_dim > 256 || c.d_vdim <= 0) return false;
+        if (c.d_conv < 1 || c.d_conv > 16) return false;
+        if (c.d_decay_channels && c.d_a_rank <= 0) return false;
+        if (c.d_gate == MI355_HYB_GATE_SIGMOID_LR && c.d_g_rank <= 0) return false;
+        if (c.d_gate != MI355_HYB_GATE_SIGMOID_LR && c.d_gate != MI355_HYB_GATE_SILU) return false;
+    }
+    if (c.mixer == MI355_HYB_MIX_MINGRU && c.g_width <= 0) return false;
+    if (c.mlp_kind < 0 || c.mlp_kind > 1 || (c.mlp_kind == 1 && c.mlp_ff <= 0)) return false;
+    return true;
+}
+
+// what a slot holds and in which type: matrices follow the model dtype, vectors and small tables are f32
+bool is_matrix(int which) {
+    switch (which) {
+        case MI355_HW_EMBED: case MI355_HW_HEAD: case MI355_HW_IN_PROJ: case MI355_HW_OUT_PROJ: case MI355_HW_D_A2: case MI355_HW_D_G2:
+        case MI355_HW_MLP_GATE_UP: case MI355_HW_MLP_DOWN: return true;
+        default: return false;
+    }
+}
+
+int64_t expected_elems(const HModel* m, int layer, int which) {
+    const int W = m->cfg.width;
+    if (layer < 0) {
+        if (which == MI355_HW_EMBED || which == MI355_HW_HEAD) return (int64_t)m->cfg.vocab * W;
+        if (which == MI355_HW_FINAL_NORM) return W;
+        return -1;
+    }
+    const HLayer& L = m->layers[layer];
+    const mi355_hybrid_layer& c = L.c;
+    switch (which) {
+        case MI355_HW_NORM1: return W;
+        case MI355_HW_NORM2: return c.mlp_kind ? W : -1;
+        case MI355_HW_IN_PROJ: return (int64_t)L.in_rows * W;
+        case MI355_HW_IN_BIAS: return L.in_rows;
+        case MI355_HW_OUT_PROJ: return (int64_t)W * L.out_k;
+        case MI355_HW_A_QNORM: case MI355_HW_A_KNORM: return L.has_attn() && c.a_qk_norm ? c.a_dim : -1;
+        case MI355_HW_A_SINK: return L.has_attn() && c.a_has_sink ? c.a_heads : -1;
+        case MI355_HW_D_CONV: return L.has_delta() ? (int64_t)L.conv_channels() * c.d_conv : -1;
+        case MI355_HW_D_A_LOG: return L.has_delta() ? c.d_heads : -1;
+        case MI355_HW_D_DT_BIAS: return L.has_delta() ? (c.d_decay_channels ? c.d_heads * c.d_dim : c.d_heads) : -1;
+        case MI355_HW_D_NORM: return L.has_delta() ? c.d_vdim : -1;
+        case MI355_HW_D_A2: return L.has_delta() && c.d_decay_channels ? (int64_t)c.d_heads * c.d_dim * c.d_a_rank : -1;
+        case MI355_HW_D_G2: return L.has_delta() && c.d_gate == MI355_HYB_GATE_SIGMOID_LR ? (int64_t)c.d_heads * c.d_vdim * c.d_g_rank : -1;
+        case MI355_HW_MLP_GATE_UP: return c.mlp_kind ? (int64_t)2 * c.mlp_ff * W : -1;
+        case MI355_HW_MLP_DOWN: return c.mlp_kind ? (int64_t)W * c.mlp_ff : -1;
+        default: return -1;
+    }
+}
+
+Weight* slot_of(HModel* m, int layer, int which) {
+    if (layer < 0) return which == MI355_HW_EMBED ? &m->embed : which == MI355_HW_FINAL_NORM ? &m->final_norm : which == MI355_HW_HEAD ? &m->head : nullptr;
+    if (layer >= (int)m->layers.size() || which < MI355_HW_NORM1 || which >= MI355_HW_COUNT) return nullptr;
+    return &m->layers[layer].w[which];
+}
+
+// device bf16 bits -> the slot's storage
+int store_weight(HModel* m, int layer, int which, const uint16_t* dev_bits, int64_t n, int64_t stream) {
+    Weight* w = slot_of(m, layer, which);
+    if (!w || n != expected_elems(m, layer, which)) return -2;
+    const bool as_bf16 = is_matrix(which) && m->bf16();
+    if (w->p) { (void)hipFree(w->p); w->p = nullptr; }
+    HHIP(hipMalloc(&w->p, (size_t)n * (as_bf16 ? 2 : 4)));
+    w->n = n;
+    if (as_bf16) HHIP(hipMemcpyAsync(w->p, dev_bits, (size_t)n * 2, hipMemcpyDeviceToDevice, reinterpret_cast<hipStream_t>(stream)));
+    else HCHECK(mi355_hyb_bf16_to_f32(static_cast<float*>(w->p), dev_bits, n, stream));
+    return 0;
+}
+
+template <typename T> int grow(T*& p, size_t bytes) {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    void* q = nullptr;
+    const hipError_t e = hipMalloc(&q, bytes ? bytes : 16);
+    if (e != hipSuccess) return (int)e;
+    p = static_cast<T*>(q);
+    return 0;
+}
+
+int ensure_capacity(HModel* m, int T, int n_out) {
+    if (T > m->cap_t) {
+        const size_t t = (size_t)T, W = (size_t)m->cfg.width;
+        HHIP(hipDeviceSynchronize());
+        HCHECK(grow(m->x, t * W * 4));
+        HCHECK(grow(m->proj, t * m->max_in_rows * 4));
+        HCHECK(grow(m->aux1, t * (size_t)m->max_aux1 * 4));
+        HCHECK(grow(m->aux2, t * (size_t)m->max_aux2 * 4));
+        HCHECK(grow(m->conv, t * (size_t)m->max_conv * 4));
+        HCHECK(grow(m->o, t * (size_t)m->max_o * 4));
+        HCHECK(grow(m->y, t * W * 4));
+        HCHECK(grow(m->gu, t * (size_t)m->max_ff * 2 * 4));
+        HCHECK(grow(m->xcopy, t * W * 2));
+        HCHECK(grow(m->q, t * (size_t)m->max_q * m->esize()));
+        HCHECK(grow(m->mix, t * (size_t)m->max_mix * m->esize()));
+        HCHECK(grow(m->act, t * (size_t)m->max_ff * m->esize()));
+        HCHECK(grow(m->tok_seq, t * 4));
+        m->cap_t = T;
+    }
+    if (n_out > m->cap_out) {
+        HHIP(hipDeviceSynchronize());
+        HCHECK(grow(m->xn, (size_t)n_out * m->cfg.width * m->esize()));
+        m->cap_out = n_out;
+    }
+    return 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t mi355_hybrid_in_proj_rows(const mi355_hybrid_layer* layer, int32_t* offsets) {
+    int32_t off[P_COUNT];
+    if (!layer) return -1;
+    const int r = in_proj_parts(*layer, off);
+    if (offsets) std::memcpy(offsets, off, sizeof(off));
+    return r;
+}
+
+void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_layer* layers) {
+    if (!cfg || !layers || cfg->width <= 0 || cfg->vocab <= 0 || cfg->n_layers <= 0 || cfg->block_size <= 0 || cfg->state_slots <= 0) return nullptr;
+    if (cfg->dtype != MI355_DTYPE_F32 && cfg->dtype != MI355_DTYPE_BF16) return nullptr;
+    for (int i = 0; i < cfg->n_layers; ++i) if (!layer_ok(layers[i])) return nullptr;
+    HModel* m = new HModel();
+    m->cfg = *cfg;
+    m->layers.resize(cfg->n_layers);
+    int64_t off = 0;
+    for (int i = 0; i < cfg->n_layers; ++i) {
+        HLayer& L = m->layers[i];
+        L.c = layers[i];
+        const mi355_hybrid_layer& c = L.c;
+        L.in_rows = in_proj_parts(c, L.off);
+        L.out_k = 0;
+        if (L.has_attn()) L.out_k += c.a_heads * c.a_vdim;
+        if (L.has_delta()) L.out_k += c.d_heads * c.d_vdim;
+        if (c.mixer == MI355_HYB_MIX_MINGRU) L.out_k = c.g_width;
+        m->max_in_rows = std::max(m->max_in_rows, L.in_rows);
+        m->max_mix = std::max(m->max_mix, L.out_k);
+        if (L.has_attn()) m->max_q = std::max(m->max_q, c.a_heads * c.a_dim);
+        if (L.has_delta()) {
+            if (c.d_decay_channels) m->max_aux1 = std::max(m->max_aux1, c.d_heads * c.d_dim);
+            if (c.d_gate == MI355_HYB_GATE_SIGMOID_LR) m->max_aux2 = std::max(m->max_aux2, c.d_heads * c.d_vdim);
+            m->max_conv = std::max(m->max_conv, L.conv_channels());
+            m->max_o = std::max(m->max_o, c.d_heads * c.d_vdim);
+            L.conv_off = off; off += (int64_t)L.conv_channels() * (c.d_conv - 1);
+            L.state_off = off; off += (int64_t)c.d_heads * c.d_dim * c.d_vdim;
+        }
+        if (c.mixer == MI355_HYB_MIX_MINGRU) { L.state_off = off; off += c.g_width; }
+        if (c.mlp_kind) m->max_ff = std::max(m->max_ff, c.mlp_ff);
+    }
+    m->slot_floats = std::max<int64_t>(off, 1);
+    return m;
+}
+
+void mi355_hybrid_destroy(void* mp) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m) return;
+    (void)hipDeviceSynchronize();
+    for (HLayer& L : m->layers) {
+        for (Weight& w : L.w) if (w.p) (void)hipFree(w.p);
+        for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.k_pages, L.v_pages}) if (p) (void)hipFree(p);
+    }
+    for (void* p : {m->embed.p, m->final_norm.p, m->head.p, (void*)m->state, (void*)m->x, (void*)m->proj, (void*)m->aux1, (void*)m->aux2,
+                    (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, (void*)m->tok_seq})
+        if (p) (void)hipFree(p);
+    delete m;
+}
+
+int mi355_hybrid_set_weight(void* mp, int32_t layer, int32_t which, const uint16_t* host_bf16, int64_t n) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m || !host_bf16 || n <= 0) return -1;
+    if (n != expected_elems(m, layer, which)) return -2;
+    uint16_t* tmp = nullptr;
+    HHIP(hipMalloc(reinterpret_cast<void**>(&tmp), (size_t)n * 2));
+    int rc = (int)hipMemcpy(tmp, host_bf16, (size_t)n * 2, hipMemcpyHostToDevice);
+    if (rc == 0) rc = store_weight(m, layer, which, tmp, n, 0);
+    if (rc == 0) rc = (int)hipDeviceSynchronize();
+    (void)hipFree(tmp);
+    return rc;
+}
+
+int mi355_hybrid_set_weight_dev(void* mp, int32_t layer, int32_t which, const uint16_t* dev_bf16, int64_t n, int64_t stream) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m || !dev_bf16 || n <= 0) return -1;
+    return store_weight(m, layer, which, dev_bf16, n, stream);
+}
+
+int mi355_hybrid_set_rope_tables(void* mp, int32_t layer, const float* cos_t, const float* sin_t, int32_t n_positions) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m || layer < 0 || layer >= (int)m->layers.size() || !cos_t || !sin_t || n_positions <= 0) return -1;
+    HLayer& L = m->layers[layer];
+    if (!L.has_attn() || L.c.a_rot_dims <= 0) return -2;
+    const size_t bytes = (size_t)n_positions * (L.c.a_rot_dims / 2) * 4;
+    HHIP(hipDeviceSynchronize());
+    HCHECK(grow(L.cos_t, bytes));
+    HCHECK(grow(L.sin_t, bytes));
+    HHIP(hipMemcpy(L.cos_t, cos_t, bytes, hipMemcpyHostToDevice));
+    HHIP(hipMemcpy(L.sin_t, sin_t, bytes, hipMemcpyHostToDevice));
+    L.n_pos = n_positions;
+    return 0;
+}
+
+int64_t mi355_hybrid_state_floats_per_slot(void* mp) { return mp ? static_cast<HModel*>(mp)->slot_floats : -1; }
+void* mi355_hybrid_state_ptr(void* mp) { return mp ? static_cast<HModel*>(mp)->state : nullptr; }
+
+int64_t mi355_hybrid_cache_bytes(void* mp, int32_t num_blocks) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m || num_blocks < 0) return -1;
+    int64_t b = m->slot_floats * 4 * m->cfg.state_slots;
+    for (const HLayer& L : m->layers)
+        if (L.has_attn()) b += (int64_t)num_blocks * m->cfg.block_size * L.c.a_kv_heads * (L.c.a_dim + L.c.a_vdim) * (int64_t)m->esize();
+    return b;
+}
+
+int mi355_hybrid_alloc_cache(void* mp, int32_t num_blocks) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m || num_blocks <= 0) return -1;
+    HHIP(hipDeviceSynchronize());
+    for (HLayer& L : m->layers) {
+        if (!L.has_attn()) continue;
+        const size_t rows = (size_t)num_blocks * m->cfg.block_size * L.c.a_kv_heads;
+        HCHECK(grow(L.k_pages, rows * L.c.a_dim * m->esize()));
+        HCHECK(grow(L.v_pages, rows * L.c.a_vdim * m->esize()));
+        HHIP(hipMemset(L.k_pages, 0, rows * L.c.a_dim * m->esize()));
+        HHIP(hipMemset(L.v_pages, 0, rows * L.c.a_vdim * m->esize()));
+    }
+    const size_t sb = (size_t)m->slot_floats * 4 * m->cfg.state_slots;
+    HCHECK(grow(m->state, sb));
+    HHIP(hipMemset(m->state, 0, sb));
+    HHIP(hipDeviceSynchronize());
+    m->num_blocks = num_blocks;
+    return 0;
+}
+
+int mi355_hybrid_forward(void* mp, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+                         const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                         const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t T,
+                         int32_t max_blocks, int32_t max_context_len, float* logits, float* layer_trace, int64_t stream) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (!m || !tokens || !positions || !slot_mapping || !block_tables || !context_lens || !cu_seqlens_q || !state_slots) return -1;
+    if (num_seqs <= 0 || T <= 0 || n_out < 0 || (n_out > 0 && (!out_rows || !logits)) || max_blocks <= 0) return -1;
+    if (!m->state || !m->embed.p || !m->final_norm.p || !m->head.p) return -3;
+    if ((int64_t)max_blocks * m->cfg.block_size < max_context_len) return -4;
+    for (const HLayer& L : m->layers) {
+        const int need[] = {MI355_HW_NORM1, MI355_HW_IN_PROJ, MI355_HW_OUT_PROJ};
+        for (int s : need) if (!L.w[s].p) return -3;
+        for (int s = MI355_HW_NORM2; s < MI355_HW_COUNT; ++s)
+            if (s != MI355_HW_IN_BIAS && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
+        if (L.has_attn() && (!L.k_pages || (L.c.a_rot_dims > 0 && L.n_pos < max_context_len))) return -4;
+    }
+    HCHECK(ensure_capacity(m, T, n_out));
+    const int W = m->cfg.width, dt = m->cfg.dtype;
+    const float eps = m->cfg.norm_eps;
+    const bool bf = m->bf16();
+    void* xin = bf ? m->xcopy : (void*)m->x;                       // what the sublayers' first product reads
+    const int xin_dt = bf ? MI355_DTYPE_BF16 : MI355_DTYPE_F32;
+    HCHECK(mi355_hyb_token_seq(m->tok_seq, cu_seqlens_q, num_seqs, stream));
+    HCHECK(mi355_hyb_embed(m->x, bf ? m->xcopy : nullptr, m->embed.p, tokens, T, W, m->cfg.vocab, dt, stream));
+    for (size_t li = 0; li < m->layers.size(); ++li) {
+        HLayer& L = m->layers[li];
+        const mi355_hybrid_layer& c = L.c;
+        auto f = [&](int which) { return static_cast<const float*>(L.w[which].p); };
+        const int ldp = L.in_rows;
+        HCHECK(mi355_hyb_linear(m->proj, ldp, xin, xin_dt, W, L.w[MI355_HW_IN_PROJ].p, f(MI355_HW_IN_BIAS), T, L.in_rows, W, dt, stream));
+        int mix_col = 0;
+        if (L.has_attn()) {
+            HCHECK(mi355_hyb_attn_prepare(m->q, L.k_pages, L.v_pages, m->proj, ldp, L.off[P_AQ], L.off[P_AK], L.off[P_AV],
+                                          c.a_qk_norm ? f(MI355_HW_A_QNORM) : nullptr, c.a_qk_norm ? f(MI355_HW_A_KNORM) : nullptr,
+                                          L.cos_t, L.sin_t, positions, slot_mapping, T, c.a_heads, c.a_kv_heads, c.a_dim, c.a_vdim,
+                                          c.a_rot_dims, eps, dt, stream));
+            HCHECK(mi355_hyb_window_attention(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens, cu_seqlens_q,
+                                              m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, c.a_heads,
+                                              c.a_kv_heads, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window, c.a_scale,
+                                              c.mixer == MI355_HYB_MIX_PARALLEL ? c.a_out_scale : 1.f, dt, stream));
+            mix_col = c.a_heads * c.a_vdim;
+        }
+        if (L.has_delta()) {
+            const int C = L.conv_channels();
+            float* conv_state = m->state + L.conv_off;
+            HCHECK(mi355_hyb_conv_silu(m->conv, m->proj, ldp, L.off[P_DQ], f(MI355_HW_D_CONV), conv_state, m->slot_floats, context_lens,
+                                       cu_seqlens_q, state_slots, m->tok_seq, num_seqs, T, C, c.d_conv, stream));
+            HCHECK(mi355_hyb_conv_state_update(conv_state, m->slot_floats, m->proj, ldp, L.off[P_DQ], context_lens, cu_seqlens_q,
+                                               state_slots, num_seqs, C, c.d_conv, stream));
+            const float* decay_in = m->proj + L.off[P_A];
+            int ldd = ldp;
+            if (c.d_decay_channels) {
+                HCHECK(mi355_hyb_linear(m->aux1, c.d_heads * c.d_dim, m->proj + L.off[P_A], MI355_DTYPE_F32, ldp, L.w[MI355_HW_D_A2].p,
+                                        nullptr, T, c.d_heads * c.d_dim, c.d_a_rank, dt, stream));
+                decay_in = m->aux1; ldd = c.d_heads * c.d_dim;
+            }
+            const float* gate_in = m->proj + L.off[P_G];
+            int ldg = ldp;
+            if (c.d_gate == MI355_HYB_GATE_SIGMOID_LR) {
+                HCHECK(mi355_hyb_linear(m->aux2, c.d_heads * c.d_vdim, m->proj + L.off[P_G], MI355_DTYPE_F32, ldp, L.w[MI355_HW_D_G2].p,
+                                        nullptr, T, c.d_heads * c.d_vdim, c.d_g_rank, dt, stream));
+                gate_in = m->aux2; ldg = c.d_heads * c.d_vdim;
+            }
+            HCHECK(mi355_hyb_delta_rule(m->o, m->state + L.state_off, m->slot_floats, m->conv, C, m->proj, ldp, L.off[P_B], decay_in, ldd,
+                                        c.d_decay_channels, f(MI355_HW_D_A_LOG), f(MI355_HW_D_DT_BIAS), context_lens, cu_seqlens_q,
+                                        state_slots, num_seqs, c.d_heads, c.d_kv_heads, c.d_dim, c.d_vdim, m->cfg.unit_eps, stream));
+            HCHECK(mi355_hyb_gated_norm(m->mix, dt, L.out_k, mix_col, m->o, f(MI355_HW_D_NORM), gate_in, ldg, c.d_gate, T, c.d_heads,
+                                        c.d_vdim, eps, c.mixer == MI355_HYB_MIX_PARALLEL ? c.d_out_scale : 1.f, stream));
+        }
+        if (c.mixer == MI355_HYB_MIX_MINGRU)
+            HCHECK(mi355_hyb_mingru(m->mix, dt, m->state + L.state_off, m->slot_floats, m->proj, ldp, L.off[0], L.off[1], L.off[2],
+                                    context_lens, cu_seqlens_q, state_slots, num_seqs, c.g_width, stream));
+        HCHECK(mi355_hyb_linear(m->y, W, m->mix, dt, L.out_k, L.w[MI355_HW_OUT_PROJ].p, nullptr, T, W, L.out_k, dt, stream));
+        HCHECK(mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(MI355_HW_NORM1), T, W, eps, stream));
+        if (c.mlp_kind) {
+            HCHECK(mi355_hyb_linear(m->gu, 2 * c.mlp_ff, xin, xin_dt, W, L.w[MI355_HW_MLP_GATE_UP].p, nullptr, T, 2 * c.mlp_ff, W, dt, stream));
+            HCHECK(mi355_hyb_clamped_glu(m->act, dt, m->gu, T, c.mlp_ff, c.mlp_limit, c.mlp_alpha, stream));
+            HCHECK(mi355_hyb_linear(m->y, W, m->act, dt, c.mlp_ff, L.w[MI355_HW_MLP_DOWN].p, nullptr, T, W, c.mlp_ff, dt, stream));
+            HCHECK(mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(MI355_HW_NORM2), T, W, eps, stream));
+        }
+        if (layer_trace)
+            HHIP(hipMemcpyAsync(layer_trace + li * (size_t)T * W, m->x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, reinterpret_cast<hipStream_t>(stream)));
+    }
+    if (n_out > 0) {
+        HCHECK(mi355_hyb_gather_norm(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W, eps, stream));
+        HCHECK(mi355_hyb_linear(logits, m->cfg.vocab, m->xn, dt, W, m->head.p, nullptr, n_out, m->cfg.vocab, W, dt, stream));
+    }
+    return 0;
+}
+
+}  // extern "C"

@@ -8,6 +8,7 @@
 #include <vector>
 
 #include "../../include/mi355_vllm.h"
+#include "../../include/mi355_hybrid.h"
 
 namespace {
 
@@ -142,12 +143,47 @@ extern "C" int mi355_rope_tables(float* cos_out, float* sin_out, int32_t rotary_
 }
 
 // ABI guard: struct sizes as this build of the header sees them (hand-written mirrors compare against it)
+// The same tables with frequencies, angles and their cosines / sines taken in f64 and rounded once: for host layers whose angles are
+// not tied to the reference's f32 arithmetic (include/mi355_hybrid.h).  Default, linear and llama3 scaling.
+extern "C" int mi355_rope_tables_f64(float* cos_out, float* sin_out, int32_t rotary_dim, int32_t n_positions, double rope_theta,
+                                     const mi355_rope_scaling* sc, int32_t max_seq_len, int32_t max_position_embeddings) {
+    if (!cos_out || !sin_out || rotary_dim <= 0 || (rotary_dim & 1) || n_positions <= 0 || rope_theta <= 0) return 1;
+    const int type = sc ? sc->type : MI355_ROPE_DEFAULT;
+    if (type != MI355_ROPE_DEFAULT && type != MI355_ROPE_LINEAR && type != MI355_ROPE_LLAMA3) return 1;
+    const int half = rotary_dim / 2;
+    std::vector<double> f(half);
+    for (int i = 0; i < half; ++i) f[i] = pow(rope_theta, -2.0 * (double)i / (double)rotary_dim);
+    double pos_div = 1.0;
+    if (type == MI355_ROPE_LINEAR) { if (sc->factor <= 0) return 1; pos_div = sc->factor; }
+    if (type == MI355_ROPE_LLAMA3) {
+        if (sc->factor <= 0 || sc->low_freq_factor <= 0 || sc->high_freq_factor <= 0 || sc->high_freq_factor == sc->low_freq_factor) return 1;
+        const double orig = original_max(sc, max_position_embeddings, max_seq_len);
+        const double low_wl = orig / sc->low_freq_factor, high_wl = orig / sc->high_freq_factor;
+        for (double& freq : f) {
+            const double wavelen = 2.0 * M_PI / freq;
+            if (wavelen < high_wl) continue;
+            if (wavelen > low_wl) { freq /= sc->factor; continue; }
+            const double smooth = (orig / wavelen - sc->low_freq_factor) / (sc->high_freq_factor - sc->low_freq_factor);
+            freq = (1.0 - smooth) * freq / sc->factor + smooth * freq;
+        }
+    }
+    for (int p = 0; p < n_positions; ++p)
+        for (int i = 0; i < half; ++i) {
+            const double th = (double)p / pos_div * f[i];
+            cos_out[(size_t)p * half + i] = (float)cos(th);
+            sin_out[(size_t)p * half + i] = (float)sin(th);
+        }
+    return 0;
+}
+
 extern "C" int64_t mi355_abi_struct_size(int32_t which) {
     switch (which) {
         case 0: return (int64_t)sizeof(mi355_qmm_desc);
         case 1: return (int64_t)sizeof(mi355_llama_config);
         case 2: return (int64_t)sizeof(mi355_dense_config);
         case 3: return (int64_t)sizeof(mi355_rope_scaling);
+        case 4: return (int64_t)sizeof(mi355_hybrid_config);
+        case 5: return (int64_t)sizeof(mi355_hybrid_layer);
         default: return -1;
     }
 }

@@ -1,0 +1,286 @@
+"""Python harness over the `mi355_hybrid_*` handle (include/mi355_hybrid.h): layer-list models whose layers mix tokens by
+sliding-window attention with a sink, a gated delta rule, a minGRU, or attention and delta rule side by side.  The Sogodra design
+is read here: its config.json (`architecture`, `layers`, `norm`, `vocab`, `width`) becomes the C structs, its tensors are
+concatenated into the host layer's slots.  No CPU fallback; torch only holds device buffers."""
+import ctypes
+import json
+import os
+import struct
+
+import numpy as np
+import torch
+
+from ._lib import lib, HybridConfig, HybridLayer, RopeScaling
+
+DT_F32, DT_BF16 = 0, 2
+MIX_PARALLEL, MIX_MINGRU, MIX_DELTA, MIX_ATTENTION = 0, 1, 2, 3
+GATE_SILU, GATE_SIGMOID_LR = 0, 1
+ROPE_DEFAULT, ROPE_LLAMA3 = 0, 2
+(HW_EMBED, HW_FINAL_NORM, HW_HEAD, HW_NORM1, HW_NORM2, HW_IN_PROJ, HW_IN_BIAS, HW_OUT_PROJ, HW_A_QNORM, HW_A_KNORM, HW_A_SINK, HW_D_CONV,
+ HW_D_A_LOG, HW_D_DT_BIAS, HW_D_NORM, HW_D_A2, HW_D_G2, HW_MLP_GATE_UP, HW_MLP_DOWN) = range(19)
+
+# constants the Sogodra design fixes
+SOGODRA_GLU_ALPHA = 1.702          # y = g sigmoid(1.702 g) (u + 1)
+SOGODRA_UNIT_EPS = 1e-6            # inside the root of the unit norm of the delta rule's q and k
+DEFAULT_BLOCK_SIZE = 64
+
+
+def _check(rc, what):
+    if rc != 0:
+        raise RuntimeError(f"{what} failed with code {rc}")
+
+
+def read_safetensors(path):
+    """name -> (bf16 bits as uint16 ndarray | int32 ndarray, shape).  The format: 8-byte little-endian header length, that many
+    bytes of JSON (name -> dtype, shape, data_offsets), then the data.  bf16 / f32 tensors come back as bf16 bits (f32 values must
+    be exactly representable), integer tables as int32."""
+    with open(path, "rb") as f:
+        n = struct.unpack("<Q", f.read(8))[0]
+        meta = json.loads(f.read(n))
+        base = 8 + n
+        out = {}
+        for name, info in meta.items():
+            if name == "__metadata__":
+                continue
+            lo, hi = info["data_offsets"]
+            f.seek(base + lo)
+            raw = f.read(hi - lo)
+            shape = tuple(info["shape"])
+            if info["dtype"] == "BF16":
+                a = np.frombuffer(raw, np.uint16).copy()
+            elif info["dtype"] == "F32":
+                u = np.frombuffer(raw, np.uint32)
+                if np.any(u & 0xFFFF):
+                    raise ValueError(f"{name}: f32 values that bf16 cannot hold")
+                a = (u >> 16).astype(np.uint16)
+            elif info["dtype"] == "I32":
+                a = np.frombuffer(raw, np.int32).copy()
+            else:
+                raise ValueError(f"{name}: dtype {info['dtype']} is not served")
+            if a.size != int(np.prod(shape, dtype=np.int64)):
+                raise ValueError(f"{name}: {a.size} elements for shape {shape}")
+            out[name] = (a, shape)
+    return out
+
+
+def _bf16_bits(a):
+    u = np.ascontiguousarray(a, np.float32).view(np.uint32)
+    return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+
+
+class SogodraSpec:
+    """config.json of a Sogodra model -> layer structs + the tensor names behind every weight slot"""
+
+    def __init__(self, cfg, shapes):
+        """cfg: the parsed config.json; shapes: tensor name -> shape (which optional tensors exist, ranks of low-rank parts)"""
+        if cfg.get("architecture") != "Sogodra":
+            raise ValueError("not a Sogodra config")
+        self.cfg = cfg
+        self.width, self.vocab = int(cfg["width"]), int(cfg["vocab"])
+        self.eps = float(cfg["norm"]["eps"])
+        self.layers, self.slots, self.rope = [], [], []
+        for i, lc in enumerate(cfg["layers"]):
+            L, slots, rope = self._layer("l%d." % i, lc, shapes)
+            self.layers.append(L)
+            self.slots.append(slots)
+            self.rope.append(rope)
+
+    def _attention(self, L, p, c, shapes, slots):
+        L.a_heads, L.a_kv_heads, L.a_dim, L.a_vdim = int(c["heads"]), int(c["kv_heads"]), int(c["dim"]), int(c["vdim"])
+        L.a_window = int(c["mask"]["size"]) if c.get("mask") else 0
+        rot = c.get("rot")
+        L.a_rot_dims = int(rot["dims"]) if rot else 0
+        L.a_scale = float(c["scale"])
+        L.a_has_sink = int(p + "sink" in shapes)
+        L.a_qk_norm = int(p + "q.norm" in shapes)
+        if L.a_qk_norm:
+            slots[HW_A_QNORM], slots[HW_A_KNORM] = [p + "q.norm"], [p + "k.norm"]
+        if L.a_has_sink:
+            slots[HW_A_SINK] = [p + "sink"]
+        return [p + "q", p + "k", p + "v"], [p + "o"], rot
+
+    def _delta(self, L, p, c, shapes, slots, per_channel, gate):
+        L.d_heads, L.d_kv_heads, L.d_dim, L.d_vdim, L.d_conv = (int(c["heads"]), int(c["kv_heads"]), int(c["dim"]), int(c["vdim"]),
+                                                                int(c["conv"]))
+        L.d_decay_channels, L.d_gate = int(per_channel), gate
+        a_name, g_name = ("a1" if per_channel else "a"), ("g1" if gate == GATE_SIGMOID_LR else "g")
+        if per_channel:
+            L.d_a_rank = int(shapes[p + "a1"][0])
+            slots[HW_D_A2] = [p + "a2"]
+        if gate == GATE_SIGMOID_LR:
+            L.d_g_rank = int(shapes[p + "g1"][0])
+            slots[HW_D_G2] = [p + "g2"]
+        slots[HW_D_CONV] = [p + "q.conv", p + "k.conv", p + "v.conv"]
+        slots[HW_D_A_LOG], slots[HW_D_DT_BIAS], slots[HW_D_NORM] = [p + "A_log"], [p + "dt_bias"], [p + "norm"]
+        return [p + "q", p + "k", p + "v", p + "b", p + a_name, p + g_name], [p + "o"]
+
+    def _layer(self, p, lc, shapes):
+        L, slots, rope = HybridLayer(), {HW_NORM1: [p + "norm1"]}, None
+        m, kind = lc["mixer"], lc["type"]
+        if kind == "parallel":
+            L.mixer = MIX_PARALLEL
+            ins, outs, rope = self._attention(L, p + "mix.left.", m["left"], shapes, slots)
+            i2, o2 = self._delta(L, p + "mix.right.", m["right"], shapes, slots, True, GATE_SIGMOID_LR)
+            ins, outs = ins + i2, outs + o2
+            L.a_out_scale, L.d_out_scale = float(m["left_scale"]), float(m["right_scale"])
+        elif kind == "delta":
+            L.mixer = MIX_DELTA
+            ins, outs = self._delta(L, p + "mix.", m, shapes, slots, False, GATE_SILU)
+            L.d_out_scale = 1.0
+        elif kind == "mingru":
+            L.mixer = MIX_MINGRU
+            L.g_width = int(m["width"])
+            ins, outs = [p + "mix.z", p + "mix.x", p + "mix.g"], [p + "mix.o"]
+            slots[HW_IN_BIAS] = [p + "mix.z.b", p + "mix.x.b", None]
+        else:
+            raise ValueError(f"layer type {kind!r} is not part of the design")
+        slots[HW_IN_PROJ], slots[HW_OUT_PROJ] = ins, outs
+        mlp = lc.get("mlp")
+        if mlp:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not part of the design")
+            L.mlp_kind, L.mlp_ff, L.mlp_limit, L.mlp_alpha = 1, int(mlp["ff"]), float(mlp["limit"]), SOGODRA_GLU_ALPHA
+            slots[HW_NORM2] = [p + "norm2"]
+            slots[HW_MLP_GATE_UP], slots[HW_MLP_DOWN] = [p + "mlp.gate", p + "mlp.up"], [p + "mlp.down"]
+        return L, slots, rope
+
+
+class HybridModel:
+    stateful = True                       # its layers carry state from token to token: a sequence needs a state slot
+
+    def __init__(self, spec, dtype="bfloat16", block_size=DEFAULT_BLOCK_SIZE, state_slots=4):
+        self.spec, self.block_size, self.state_slots = spec, int(block_size), int(state_slots)
+        self.dtype = {"bfloat16": DT_BF16, "bf16": DT_BF16, "float32": DT_F32, "f32": DT_F32}[dtype]
+        self.vocab, self.width = spec.vocab, spec.width
+        n = len(spec.layers)
+        self._layers = (HybridLayer * n)(*spec.layers)
+        c = HybridConfig(width=spec.width, vocab=spec.vocab, n_layers=n, dtype=self.dtype, block_size=self.block_size,
+                         state_slots=self.state_slots, norm_eps=spec.eps, unit_eps=SOGODRA_UNIT_EPS)
+        self.h = lib.mi355_hybrid_create(ctypes.byref(c), self._layers)
+        if not self.h:
+            raise RuntimeError("mi355_hybrid_create refused the configuration")
+        self.rope_positions = 0
+        self.num_blocks = 0
+
+    def __del__(self):
+        if getattr(self, "h", None) and lib is not None:
+            lib.mi355_hybrid_destroy(self.h)
+            self.h = None
+
+    # ---- weights
+    @classmethod
+    def from_pretrained(cls, model_dir, dtype="bfloat16", block_size=DEFAULT_BLOCK_SIZE, state_slots=4):
+        cfg = json.load(open(os.path.join(model_dir, "config.json")))
+        tensors = read_safetensors(os.path.join(model_dir, "model.safetensors"))
+        spec = SogodraSpec(cfg, {k: v[1] for k, v in tensors.items()})
+        m = cls(spec, dtype=dtype, block_size=block_size, state_slots=state_slots)
+        m.load_tensors({k: v[0] for k, v in tensors.items()}, {k: v[1] for k, v in tensors.items()})
+        return m
+
+    def _put(self, layer, which, bits):
+        bits = np.ascontiguousarray(bits, np.uint16).reshape(-1)
+        _check(lib.mi355_hybrid_set_weight(self.h, layer, which, bits.ctypes.data, bits.size), f"set_weight layer {layer} slot {which}")
+
+    def load_tensors(self, bits, shapes):
+        """bits: tensor name -> bf16 bits (uint16, any shape); shapes: name -> shape.  Concatenates what the host layer keeps as one
+        matrix: the input projections along the rows, the output projections along k."""
+        spec = self.spec
+        for which, name in ((HW_EMBED, "embed"), (HW_FINAL_NORM, "final.norm"), (HW_HEAD, "head")):
+            self._put(-1, which, bits[name])
+        for i, slots in enumerate(spec.slots):
+            for which, names in slots.items():
+                if which == HW_IN_BIAS:
+                    offs = (ctypes.c_int32 * 9)()
+                    rows = lib.mi355_hybrid_in_proj_rows(ctypes.byref(self._layers[i]), offs)
+                    parts, total = [], 0
+                    for nm, proj in zip(names, slots[HW_IN_PROJ]):
+                        r = int(shapes[proj][0])
+                        parts.append(np.asarray(bits[nm], np.uint16).reshape(-1) if nm else np.zeros(r, np.uint16))
+                        total += r
+                    assert total == rows
+                    self._put(i, which, np.concatenate(parts))
+                elif which == HW_OUT_PROJ and len(names) > 1:
+                    mats = [np.asarray(bits[nm], np.uint16).reshape(shapes[nm]) for nm in names]
+                    self._put(i, which, np.concatenate(mats, axis=1))
+                elif which == HW_D_CONV:
+                    mats = [np.asarray(bits[nm], np.uint16).reshape(shapes[nm]) for nm in names]
+                    self._put(i, which, np.concatenate(mats, axis=0))
+                else:
+                    self._put(i, which, np.concatenate([np.asarray(bits[nm], np.uint16).reshape(-1) for nm in names]))
+
+    def load_state_dict_f32(self, W):
+        """W: tensor name -> f32 ndarray (tests, synthetic weights); rounded to bf16"""
+        self.load_tensors({k: _bf16_bits(v) for k, v in W.items()}, {k: tuple(np.shape(v)) for k, v in W.items()})
+
+    # ---- cache
+    def ensure_rope(self, n_positions):
+        """cos / sin tables of every attention layer up to n_positions (the framework's table builder in its f64 form; llama3 scaling when
+        the config has `rot.scaling`)"""
+        if n_positions <= self.rope_positions:
+            return
+        n = max(int(n_positions), 2 * self.rope_positions, 256)
+        for i, (L, rot) in enumerate(zip(self.spec.layers, self.spec.rope)):
+            if not rot or L.a_rot_dims <= 0:
+                continue
+            half = L.a_rot_dims // 2
+            cos, sin = np.zeros((n, half), np.float32), np.zeros((n, half), np.float32)
+            sc = rot.get("scaling")
+            rs = RopeScaling()
+            if sc:
+                rs.type, rs.factor, rs.low_freq_factor, rs.high_freq_factor = ROPE_LLAMA3, float(sc["factor"]), float(sc["low"]), float(sc["high"])
+                rs.original_max_position_embeddings = float(sc["original"])
+            else:
+                rs.type = ROPE_DEFAULT
+            _check(lib.mi355_rope_tables_f64(cos.ctypes.data, sin.ctypes.data, L.a_rot_dims, n, float(rot["base"]), ctypes.byref(rs), n, n),
+                   "rope_tables")
+            _check(lib.mi355_hybrid_set_rope_tables(self.h, i, cos.ctypes.data, sin.ctypes.data, n), "set_rope_tables")
+        self.rope_positions = n
+
+    def alloc_cache(self, num_blocks):
+        _check(lib.mi355_hybrid_alloc_cache(self.h, int(num_blocks)), "alloc_cache")
+        self.num_blocks = int(num_blocks)
+        self.ensure_rope(self.num_blocks * self.block_size)
+
+    def cache_bytes(self, num_blocks):
+        return int(lib.mi355_hybrid_cache_bytes(self.h, int(num_blocks)))
+
+    # ---- one step
+    def step(self, meta, state_slots, want_rows=None, trace=False, stream=None, sync=True):
+        """meta: BlockEngine.prepare_prompt's dict (every sequence brings its not yet cached tokens: a prompt, a portion of one, or
+        one decoded token); state_slots: the sequences' slots (BlockEngine.state_acquire); want_rows: token rows whose logits are
+        wanted (default: every sequence's last).  -> logits f32 [len(want_rows), vocab] (and the residual stream behind every layer
+        [n_layers, T, width] with trace=True)."""
+        dev = "cuda"
+        n = len(meta["context_lens"])
+        T = len(meta["input_ids"])
+        cu = np.asarray(meta["cu_seqlens_q"]).astype(np.int64)
+        if want_rows is None:
+            want_rows = (cu[1:] - 1).tolist()
+        want = np.asarray(want_rows, np.int32)
+        max_ctx = int(meta["max_context_len"])
+        self.ensure_rope(max_ctx)
+
+        def to(a, dt):
+            return torch.from_numpy(np.ascontiguousarray(np.asarray(a).astype(dt))).to(dev)
+        tok = to(np.asarray(meta["input_ids"]).astype(np.int64), np.int32)
+        pos, slots = to(meta["positions"], np.int64), to(meta["slot_mapping"], np.int64)
+        bt = to(np.asarray(meta["block_tables"]).astype(np.int64), np.int32).contiguous()
+        ctx, cuq = to(np.asarray(meta["context_lens"]).astype(np.int64), np.int32), to(cu, np.int32)
+        st = to(state_slots, np.int32)
+        if len(state_slots) != n or (len(state_slots) and (min(state_slots) < 0 or max(state_slots) >= self.state_slots)):
+            raise ValueError("every sequence of a step needs a state slot of the pool")
+        wr = to(want, np.int32) if len(want) else None
+        logits = torch.empty((len(want), self.vocab), dtype=torch.float32, device=dev)
+        tr = torch.empty((len(self.spec.layers), T, self.width), dtype=torch.float32, device=dev) if trace else None
+        s = torch.cuda.current_stream().cuda_stream if stream is None else stream
+        _check(lib.mi355_hybrid_forward(self.h, tok.data_ptr(), pos.data_ptr(), slots.data_ptr(), bt.data_ptr(), ctx.data_ptr(),
+                                        cuq.data_ptr(), st.data_ptr(), wr.data_ptr() if wr is not None else None, len(want), n, T,
+                                        bt.shape[1], max_ctx, logits.data_ptr() if len(want) else None,
+                                        tr.data_ptr() if trace else None, s), "hybrid_forward")
+        if sync:
+            torch.cuda.synchronize()
+        return (logits, tr) if trace else logits
+
+    def forward_prefill(self, meta, state_slots):
+        """logits of the last new token of every sequence (the prompt step of the engine loop)"""
+        return self.step(meta, state_slots)

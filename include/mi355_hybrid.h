@@ -1,0 +1,176 @@
+/* C ABI of the layer-list ("hybrid") host layer: decoder-only models whose config lists, layer by layer, which token mixer a
+ * layer has -- sliding-window attention with a softmax sink, a gated delta rule (recurrent matrix state), a minGRU (recurrent vector
+ * state), or attention and delta rule side by side -- and which feed-forward.  The Sogodra design is the first user.
+ *
+ * What differs from the llama-family host layers (mi355_llama_*, mi355_dense_*):
+ *   - the residual stream, norms, attention scores, decays, gates of a recurrence and the recurrent state are f32 in both dtypes;
+ *     `dtype` = MI355_DTYPE_BF16 keeps the matrices (and the K/V pages) in bf16 and multiplies on the matrix cores with f32
+ *     accumulation, MI355_DTYPE_F32 keeps everything in f32 and multiplies with plain f32 FMAs (no reduced-precision mode);
+ *   - one step function for prompts, portions of prompts and single decoded tokens: every sequence of a step brings
+ *     cu_seqlens_q[i+1] - cu_seqlens_q[i] new tokens behind context_lens[i] - that many cached ones (the fields of
+ *     mi355_be_prepare_prompt); K/V live in the block engine's pages, recurrent state in the block engine's state slots
+ *     (mi355_be_state_*), one slot per live sequence;
+ *   - a sequence whose portion starts at position 0 starts from zero state whatever its slot held before.
+ * Every entry point returns 0 on success (hipError_t or a negative argument error otherwise) and only enqueues work on `stream`. */
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_HYB_MIX_PARALLEL 0   /* attention ("left") and gated delta rule ("right") on the same input, outputs scaled and added */
+#define MI355_HYB_MIX_MINGRU 1
+#define MI355_HYB_MIX_DELTA 2
+#define MI355_HYB_MIX_ATTENTION 3  /* the attention branch alone */
+
+#define MI355_HYB_GATE_SILU 0      /* output gate silu(W_g h), full rank                */
+#define MI355_HYB_GATE_SIGMOID_LR 1 /* output gate sigmoid(W_g2 (W_g1 h)), low rank     */
+
+typedef struct mi355_hybrid_layer {
+    int32_t mixer;                 /* MI355_HYB_MIX_*                                                              */
+    /* attention branch */
+    int32_t a_heads, a_kv_heads, a_dim, a_vdim;
+    int32_t a_window;              /* 0 = none; else a query at position i sees keys j with 0 <= i - j < a_window  */
+    int32_t a_rot_dims;            /* leading dimensions of a head that are rotated (rotate-half pairs), 0 = none  */
+    int32_t a_has_sink;            /* the softmax denominator also holds exp(sink[head])                           */
+    int32_t a_qk_norm;             /* RMS norm of every query / key head before the rotation                       */
+    float a_scale, a_out_scale;
+    /* delta-rule branch */
+    int32_t d_heads, d_kv_heads, d_dim, d_vdim, d_conv;
+    int32_t d_decay_channels;      /* 0: one decay per head (full-rank W_a [heads, width]);
+                                      1: one per head and key channel (low rank W_a2 (W_a1 h), rank d_a_rank)      */
+    int32_t d_a_rank;
+    int32_t d_gate;                /* MI355_HYB_GATE_*                                                             */
+    int32_t d_g_rank;
+    float d_out_scale;
+    /* minGRU */
+    int32_t g_width;
+    /* feed-forward: 0 = none, 1 = dense clamped gate/up with y = g sigmoid(act_alpha g) (u + 1)                   */
+    int32_t mlp_kind, mlp_ff;
+    float mlp_limit, mlp_alpha;
+} mi355_hybrid_layer;
+
+typedef struct mi355_hybrid_config {
+    int32_t width, vocab, n_layers;
+    int32_t dtype;                 /* MI355_DTYPE_F32 or MI355_DTYPE_BF16                                          */
+    int32_t block_size;            /* tokens per K/V page                                                          */
+    int32_t state_slots;           /* recurrent-state slots (live sequences)                                       */
+    float norm_eps;
+    float unit_eps;                /* eps inside the root of the unit norm of q and k in the delta rule            */
+} mi355_hybrid_config;
+
+/* weight slots: `layer` = -1 for the three global ones */
+#define MI355_HW_EMBED 0           /* [vocab, width]                                                                */
+#define MI355_HW_FINAL_NORM 1      /* [width]                                                                       */
+#define MI355_HW_HEAD 2            /* [vocab, width]                                                                */
+#define MI355_HW_NORM1 3           /* [width]  norm on the mixer's output                                           */
+#define MI355_HW_NORM2 4           /* [width]  norm on the feed-forward's output                                    */
+#define MI355_HW_IN_PROJ 5         /* every projection that reads the mixer's input, concatenated along the rows in
+                                      the order of mi355_hybrid_in_proj_rows: [rows, width]                         */
+#define MI355_HW_IN_BIAS 6         /* [rows] or absent                                                              */
+#define MI355_HW_OUT_PROJ 7        /* [width, k]: the output projections side by side along k (attention first)     */
+#define MI355_HW_A_QNORM 8
+#define MI355_HW_A_KNORM 9
+#define MI355_HW_A_SINK 10
+#define MI355_HW_D_CONV 11         /* [q channels + k channels + v channels, taps], last column = the current token */
+#define MI355_HW_D_A_LOG 12        /* [heads]                                                                       */
+#define MI355_HW_D_DT_BIAS 13      /* [heads] or [heads * dim]                                                      */
+#define MI355_HW_D_NORM 14         /* [vdim]                                                                        */
+#define MI355_HW_D_A2 15           /* [heads * dim, a_rank]                                                         */
+#define MI355_HW_D_G2 16           /* [heads * vdim, g_rank]                                                        */
+#define MI355_HW_MLP_GATE_UP 17    /* [2 ff, width]: gate rows, then up rows                                        */
+#define MI355_HW_MLP_DOWN 18       /* [width, ff]                                                                   */
+#define MI355_HW_COUNT 19
+
+void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_layer* layers);
+void mi355_hybrid_destroy(void* model);
+/* rows of a layer's concatenated input projection, and where each part starts: parts = attention q, k, v, delta q, k, v, beta,
+ * decay (a or a1), gate (g or g1) for the attention / delta / parallel mixers; z, x, g for the minGRU.  offsets[9], -1 = absent */
+int32_t mi355_hybrid_in_proj_rows(const mi355_hybrid_layer* layer, int32_t* offsets);
+/* HOST bf16 bits (a checkpoint tensor), n elements; converted to the storage type of the slot */
+int mi355_hybrid_set_weight(void* model, int32_t layer, int32_t which, const uint16_t* host_bf16, int64_t n);
+/* DEVICE bf16 bits (synthetic weights of a benchmark) */
+int mi355_hybrid_set_weight_dev(void* model, int32_t layer, int32_t which, const uint16_t* dev_bf16, int64_t n, int64_t stream);
+/* HOST f32 [n_positions, a_rot_dims / 2] cos and sin of a layer's rotary angles (mi355_rope_tables builds them) */
+int mi355_hybrid_set_rope_tables(void* model, int32_t layer, const float* cos_t, const float* sin_t, int32_t n_positions);
+/* K/V pages of every attention layer and the state pool; all state starts as zero */
+int mi355_hybrid_alloc_cache(void* model, int32_t num_blocks);
+int64_t mi355_hybrid_cache_bytes(void* model, int32_t num_blocks);
+int64_t mi355_hybrid_state_floats_per_slot(void* model);
+void* mi355_hybrid_state_ptr(void* model);
+/* one step over DEVICE inputs.  tokens u32 [T]; positions, slot_mapping i64 [T]; block_tables u32 [num_seqs, max_blocks];
+ * context_lens u32 [num_seqs] (cached + new); cu_seqlens_q u32 [num_seqs + 1]; state_slots i32 [num_seqs]; out_rows i32 [n_out]
+ * = the token rows whose logits are wanted -> logits f32 [n_out, vocab].  layer_trace: NULL, or f32 [n_layers, T, width] that
+ * receives the residual stream behind every layer (parity hook). */
+int mi355_hybrid_forward(void* model, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+                         const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                         const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t num_tokens,
+                         int32_t max_blocks, int32_t max_context_len, float* logits, float* layer_trace, int64_t stream);
+
+/* ---- the mechanisms alone (tests, other host layers).  `dtype` is the type of 16/32-bit operands marked (dt); the rest is f32 */
+/* token_seq i32 [T]: the sequence (row of cu_seqlens_q) of every token row */
+int mi355_hyb_token_seq(int32_t* token_seq, const uint32_t* cu_seqlens_q, int32_t num_seqs, int64_t stream);
+int mi355_hyb_bf16_to_f32(float* out, const uint16_t* in, int64_t n, int64_t stream);
+int mi355_hyb_copy_f32(float* out, const float* in, int64_t n, int64_t stream);
+int mi355_hyb_fill_f32(float* out, float v, int64_t n, int64_t stream);
+/* x f32 [T, width] = table (dt) [vocab, width] rows ids; xcopy: NULL or bf16 [T, width] */
+int mi355_hyb_embed(float* x, void* xcopy, const void* table, const uint32_t* ids, int32_t num_tokens, int32_t width, int32_t vocab,
+                    int32_t dtype, int64_t stream);
+/* out (dt_out) [n_rows, width] = RMS norm with weight of the rows `rows` of x */
+int mi355_hyb_gather_norm(void* out, int32_t out_dtype, const float* x, const int32_t* rows, const float* w, int32_t n_rows,
+                          int32_t width, float eps, int64_t stream);
+/* out f32 [T, ldo] = a (dt_a: F32 or BF16) [T, lda] . w (dt) [n, k]^T + bias f32 [n] */
+int mi355_hyb_linear(float* out, int32_t ldo, const void* a, int32_t a_dtype, int32_t lda, const void* w, const float* bias,
+                     int32_t num_tokens, int32_t n, int32_t k, int32_t dtype, int64_t stream);
+/* x f32 [T, width] += y / rms(y) * w, y f32 [T, ldy]; xcopy (NULL or bf16 [T, width]) receives the rounded sum */
+int mi355_hyb_norm_add(float* x, void* xcopy, const float* y, int32_t ldy, const float* w, int32_t num_tokens, int32_t width,
+                       float eps, int64_t stream);
+/* per-head RMS norm (weights NULL = none) and rotation of q / k out of the projection rows, q -> q_out (dt) [T, heads, dim],
+ * k, v -> the pages at slot_mapping (dt), [blocks, block_size, kv_heads, dim | vdim] */
+int mi355_hyb_attn_prepare(void* q_out, void* k_pages, void* v_pages, const float* proj, int32_t ldp, int32_t q_off, int32_t k_off,
+                           int32_t v_off, const float* q_norm_w, const float* k_norm_w, const float* cos_t, const float* sin_t,
+                           const int64_t* positions, const int64_t* slot_mapping, int32_t num_tokens, int32_t heads,
+                           int32_t kv_heads, int32_t dim, int32_t vdim, int32_t rot_dims, float eps, int32_t dtype, int64_t stream);
+/* causal attention of every new token over its sequence's pages: window (0 = none), sink f32 [heads] or NULL;
+ * out (dt_out) [T, ldo] at column out_off: heads x vdim, times out_scale */
+int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                               const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                               const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, int32_t num_seqs, int32_t num_tokens,
+                               int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size, int32_t max_blocks,
+                               int32_t window, float scale, float out_scale, int32_t dtype, int64_t stream);
+/* short causal convolution over time per channel, then silu: out f32 [T, channels] from proj columns [off, off + channels);
+ * the taps - 1 inputs before a portion come from conv_state f32 [slots, channels, taps - 1] (zeros at position 0);
+ * mi355_hyb_conv_state_update then moves the state behind the portion */
+int mi355_hyb_conv_silu(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* conv_state,
+                        int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                        const int32_t* state_slots, const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t channels,
+                        int32_t taps, int64_t stream);
+int mi355_hyb_conv_state_update(float* conv_state, int64_t state_stride, const float* proj, int32_t ldp, int32_t off,
+                                const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                                int32_t num_seqs, int32_t channels, int32_t taps, int64_t stream);
+/* gated delta rule over the new tokens of every sequence, state f32 [slots] x [heads, dim, vdim] (stride in floats).
+ * qkv f32 [T, ldq]: q at 0 (kv_heads x dim, raw), k behind it, v behind that (heads x vdim); q and k are made unit vectors per head
+ * (eps inside the root), q times dim^-1/2.  beta = sigmoid(proj[:, b_off + head]).  decay = exp(-exp(a_log[head]) * softplus(da +
+ * dt_bias)) with da = decay_in[t, head] (channels = 0) or decay_in[t, head * dim + channel].  o f32 [T, heads, vdim]. */
+int mi355_hyb_delta_rule(float* o, float* state, int64_t state_stride, const float* qkv, int32_t ldq, const float* proj,
+                         int32_t ldp, int32_t b_off, const float* decay_in, int32_t ldd, int32_t decay_channels,
+                         const float* a_log, const float* dt_bias, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                         const int32_t* state_slots, int32_t num_seqs, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
+                         float unit_eps, int64_t stream);
+/* out (dt_out) [T, ldo] at out_off = o / rms(o over vdim) * w * gate(gate_in) * out_scale; gate: MI355_HYB_GATE_* (silu / sigmoid) */
+int mi355_hyb_gated_norm(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const float* o, const float* w,
+                         const float* gate_in, int32_t ldg, int32_t gate, int32_t num_tokens, int32_t heads, int32_t vdim, float eps,
+                         float out_scale, int64_t stream);
+/* minGRU over the new tokens: z = sigmoid(proj[:, z_off + c]), u = proj[:, x_off + c], candidate = u + 1/2 (u >= 0) or sigmoid(u),
+ * S = (1 - z) S + z candidate, out (dt_out) [T, width] = S silu(proj[:, g_off + c]); state f32 [slots] x [width] */
+int mi355_hyb_mingru(void* out, int32_t out_dtype, float* state, int64_t state_stride, const float* proj, int32_t ldp, int32_t z_off,
+                     int32_t x_off, int32_t g_off, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                     const int32_t* state_slots, int32_t num_seqs, int32_t width, int64_t stream);
+/* out (dt_out) [T, ff] = g sigmoid(alpha g) (u + 1), g = min(gu[:, j], limit), u = clamp(gu[:, ff + j], -limit, limit) */
+int mi355_hyb_clamped_glu(void* out, int32_t out_dtype, const float* gu, int32_t num_tokens, int32_t ff, float limit, float alpha,
+                          int64_t stream);
+
+#ifdef __cplusplus
+}
+#endif

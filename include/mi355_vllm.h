@@ -452,6 +452,9 @@ typedef struct mi355_rope_scaling {
 int32_t mi355_rope_table_len(const mi355_rope_scaling* sc, int32_t max_seq_len, int32_t max_position_embeddings);
 int mi355_rope_tables(float* cos_out_host, float* sin_out_host, int32_t rotary_dim, int32_t n_positions, double rope_theta,
                       const mi355_rope_scaling* sc /* NULL = default */, int32_t max_seq_len, int32_t max_position_embeddings);
+/* the same tables with frequencies and angles in f64, rounded once (default, linear and llama3 scaling; 1 for the others) */
+int mi355_rope_tables_f64(float* cos_out_host, float* sin_out_host, int32_t rotary_dim, int32_t n_positions, double rope_theta,
+                          const mi355_rope_scaling* sc, int32_t max_seq_len, int32_t max_position_embeddings);
 /* `Config::effective_max_seq_len` (src/openai/models/mod.rs:663-702): max(base, round(original * factor)) for yarn with
  * factor > 1, the base otherwise -- the context length the KV cache and the tables above are sized for */
 int64_t mi355_effective_max_seq_len(const mi355_rope_scaling* sc, int64_t base_max_position_embeddings);
@@ -712,6 +715,15 @@ int32_t mi355_be_prefill_chunk_blocks_required(void* be, const int64_t* seq_ids,
 int32_t mi355_be_can_append_prefill_chunk(void* be, const int64_t* seq_ids, int32_t n, int32_t chunk);
 int32_t mi355_be_append_prefill_chunk_slots(void* be, const int64_t* seq_ids, int32_t n, int32_t chunk);
 int32_t mi355_be_free_sequence(void* be, int64_t seq_id);
+/* recurrent-state slots of models whose layers carry state from token to token (include/mi355_hybrid.h): n slots in all, set once
+ * while no sequence holds one; acquire = the sequence's slot, the lowest free one at its first call (-2: none free, -1: unknown
+ * sequence); mi355_be_free_sequence gives the slot back with the blocks.  The reference keeps such state inside its model runner. */
+int32_t mi355_be_state_init(void* be, int32_t n_slots);
+int32_t mi355_be_state_acquire(void* be, int64_t seq_id);
+int32_t mi355_be_state_slot(void* be, int64_t seq_id);
+int32_t mi355_be_state_free_slots(void* be);
+/* a prompt that arrives in portions: append tokens that count as prompt (the next prompt step takes them) */
+int32_t mi355_be_seq_extend_prompt(void* be, int64_t seq_id, const uint32_t* tokens, int32_t n);
 int32_t mi355_be_cache_sequence(void* be, int64_t seq_id);
 int32_t mi355_be_evict_prefix_cache_blocks(void* be, int32_t num_blocks);
 int32_t mi355_be_evict_prefix_cache_until_free(void* be, int32_t min_free);
@@ -851,7 +863,8 @@ int mi355_llama_load_gguf_tp(const char* path, int32_t max_batch, int32_t max_bl
 int mi355_llama_check_gguf(const char* path, int32_t tp_rank, int32_t tp_world, mi355_llama_config* cfg_out);
 
 /* ABI guard for bindings that mirror the structs by hand (ctypes, a Rust #[repr(C)]): sizeof of
- * 0 = mi355_qmm_desc, 1 = mi355_llama_config, 2 = mi355_dense_config, 3 = mi355_rope_scaling; -1 for an unknown id */
+ * 0 = mi355_qmm_desc, 1 = mi355_llama_config, 2 = mi355_dense_config, 3 = mi355_rope_scaling, 4 = mi355_hybrid_config,
+ * 5 = mi355_hybrid_layer (include/mi355_hybrid.h); -1 for an unknown id */
 int64_t mi355_abi_struct_size(int32_t which);
 
 #ifdef __cplusplus
