@@ -68,6 +68,12 @@ def parse():
                          "(quick: batch 1; full: + batch 32 ragged and a 2048-token prompt step)")
     ap.add_argument("--legs", default="all", help="secondary legs at BASELINE configs[2..4] shapes on one GPU (bench_legs.py): "
                                                    "all | none | comma list of bf16_b32,gptq_qwen2,mixtral_fp8")
+    ap.add_argument("--hybrid", default="", metavar="SIZES",
+                    help="instead of the default workload: the layer-list host layer (Sogodra design, random weights) beside the 16-bit llama "
+                         "host layer at equal sizes -- comma list of 1b,3b,8b (bench_hybrid.py); prints its own JSON line")
+    ap.add_argument("--hybrid-prompt", type=int, default=2048, help="--hybrid: tokens of the prompt step")
+    ap.add_argument("--hybrid-batch", type=int, default=8, help="--hybrid: sequences of the decode steps")
+    ap.add_argument("--hybrid-ctx", type=int, default=2048, help="--hybrid: cached tokens behind every decoding sequence")
     ap.add_argument("--layers", type=int, default=0, help="debug only: fewer layers (result marked invalid)")
     ap.add_argument("--same-device", action="store_true",
                     help="rehearsal of the N > 1 command on a one-GPU box: every rank on cuda:0 (gloo control plane, the one-shot peer kernel "
@@ -441,6 +447,9 @@ def setup_comm(gm, M, dist, args, rank, world):
 
 def main():
     args = parse()
+    if args.hybrid:
+        import bench_hybrid
+        return bench_hybrid.main(args.hybrid, args.hybrid_prompt, args.hybrid_batch, args.hybrid_ctx)
     rank = int(os.environ.get("RANK", "0"))
     local_rank = int(os.environ.get("LOCAL_RANK", "0"))
     world = int(os.environ.get("WORLD_SIZE", "1"))

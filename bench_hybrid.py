@@ -1,0 +1,195 @@
+"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, random weights) at layer
+sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
+width, depth, head geometry, feed-forward size and vocabulary.  One GPU, bf16, synthetic data.  The default workload of bench.py and
+its one-line contract are not touched: this option prints its own JSON line.
+
+Per size: one prompt step of T tokens (tokens/s) and decode steps of B sequences behind `ctx` cached tokens (tokens/s), both models
+driven eagerly through their step function with device-resident inputs; the hybrid model's recurrent layers have no counterpart in
+the llama model, so the line also carries each model's weight bytes and the decode steps' achieved GB/s over them."""
+import json
+import time
+
+import numpy as np
+
+SIZES = {
+    # name: width, heads x dim (kv heads), ff, vocab, window, delta heads x dim x vdim, gru width, layers (p = parallel, g = minGRU, d = delta)
+    "1b": dict(width=2048, heads=16, kv=4, dim=128, ff=8192, vocab=32000, window=1024, dheads=16, ddim=128, dvdim=128, gru=4096, layers="pgdp"),
+    "3b": dict(width=3072, heads=24, kv=8, dim=128, ff=8192, vocab=32000, window=2048, dheads=24, ddim=128, dvdim=128, gru=6144, layers="pgdp"),
+    "8b": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, vocab=32000, window=4096, dheads=32, ddim=128, dvdim=128, gru=8192, layers="pgdp"),
+}
+
+
+def sogodra_config(s):
+    att = {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv"], "vdim": s["dim"], "scale": s["dim"] ** -0.5, "mask": {"size": s["window"]},
+           "rot": {"base": 500000.0, "dims": s["dim"], "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    right = {"conv": 4, "dim": s["ddim"], "heads": s["dheads"], "kv_heads": s["dheads"], "vdim": s["dvdim"]}
+    mlp = {"ff": s["ff"], "kind": "dense", "limit": 7.0}
+    kinds = {"p": lambda: {"type": "parallel", "mixer": {"left": att, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": mlp},
+             "g": lambda: {"type": "mingru", "mixer": {"width": s["gru"]}, "mlp": mlp},
+             "d": lambda: {"type": "delta", "mixer": right, "mlp": mlp}}
+    return {"architecture": "Sogodra", "layers": [kinds[c]() for c in s["layers"]], "norm": {"eps": 1e-5}, "vocab": s["vocab"], "width": s["width"]}
+
+
+def sogodra_shapes(cfg, a_rank=64, g_rank=64):
+    """tensor name -> shape for a config (the low-rank parts' ranks are free: the design reads them from the tensors)"""
+    W, sh = cfg["width"], {}
+    sh["embed"], sh["final.norm"], sh["head"] = (cfg["vocab"], W), (W,), (cfg["vocab"], W)
+
+    def delta(p, c, lr):
+        H, G, d, vd, t = c["heads"], c["kv_heads"], c["dim"], c["vdim"], c["conv"]
+        for n, r in (("q", G * d), ("k", G * d), ("v", H * vd)):
+            sh[p + n], sh[p + n + ".conv"] = (r, W), (r, t)
+        sh[p + "b"], sh[p + "A_log"], sh[p + "norm"], sh[p + "o"] = (H, W), (H,), (vd,), (W, H * vd)
+        if lr:
+            sh[p + "a1"], sh[p + "a2"], sh[p + "dt_bias"], sh[p + "g1"], sh[p + "g2"] = (a_rank, W), (H * d, a_rank), (H * d,), (g_rank, W), (H * vd, g_rank)
+        else:
+            sh[p + "a"], sh[p + "dt_bias"], sh[p + "g"] = (H, W), (H,), (H * vd, W)
+    for i, lc in enumerate(cfg["layers"]):
+        p, m = "l%d." % i, lc["mixer"]
+        sh[p + "norm1"] = (W,)
+        if lc["type"] == "parallel":
+            c, q = m["left"], p + "mix.left."
+            sh[q + "q"], sh[q + "k"], sh[q + "v"] = (c["heads"] * c["dim"], W), (c["kv_heads"] * c["dim"], W), (c["kv_heads"] * c["vdim"], W)
+            sh[q + "q.norm"], sh[q + "k.norm"], sh[q + "sink"], sh[q + "o"] = (c["dim"],), (c["dim"],), (c["heads"],), (W, c["heads"] * c["vdim"])
+            delta(p + "mix.right.", m["right"], True)
+        elif lc["type"] == "delta":
+            delta(p + "mix.", m, False)
+        else:
+            w = m["width"]
+            for n in ("z", "x", "g"):
+                sh[p + "mix." + n] = (w, W)
+            sh[p + "mix.z.b"], sh[p + "mix.x.b"], sh[p + "mix.o"] = (w,), (w,), (W, w)
+        if lc.get("mlp"):
+            ff = lc["mlp"]["ff"]
+            sh[p + "norm2"], sh[p + "mlp.gate"], sh[p + "mlp.up"], sh[p + "mlp.down"] = (W,), (ff, W), (ff, W), (W, ff)
+    return sh
+
+
+def build_hybrid(cfg, max_tokens, slots):
+    """random weights generated on the GPU, concatenated as the loader does it, handed over as device bf16"""
+    import torch
+    from candle_vllm_amd import hybrid_model as hm
+    shapes = sogodra_shapes(cfg)
+    spec = hm.SogodraSpec(cfg, shapes)
+    m = hm.HybridModel(spec, dtype="bfloat16", block_size=64, state_slots=slots)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    nbytes = 0
+
+    def rnd(shape, name):
+        fan = shape[-1] if len(shape) > 1 else 1
+        if name.endswith("norm") or name.endswith("norm1") or name.endswith("norm2"):
+            return (1 + 0.02 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
+        if name == "embed":
+            return torch.randn(shape, generator=g, device="cuda").to(torch.bfloat16)
+        s = 0.5 if name.endswith(".conv") else (fan ** -0.5 if len(shape) > 1 else 0.3)
+        return (s * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
+
+    def put(layer, which, names, axis=0):
+        nonlocal nbytes
+        ts = [rnd(shapes[n], n) if n else None for n in names]
+        if which == hm.HW_IN_BIAS:
+            rows = [shapes[p][0] for p in spec.slots[layer][hm.HW_IN_PROJ]]
+            ts = [t if t is not None else torch.zeros(r, dtype=torch.bfloat16, device="cuda") for t, r in zip(ts, rows)]
+        t = torch.cat([x if axis else x.reshape(-1) for x in ts], dim=1 if axis else 0).contiguous()
+        nbytes += t.numel() * 2
+        hm._check(hm.lib.mi355_hybrid_set_weight_dev(m.h, layer, which, t.data_ptr(), t.numel(), torch.cuda.current_stream().cuda_stream), "set_weight_dev")
+        torch.cuda.synchronize()
+    for which, name in ((hm.HW_EMBED, "embed"), (hm.HW_FINAL_NORM, "final.norm"), (hm.HW_HEAD, "head")):
+        put(-1, which, [name])
+    for i, slots_ in enumerate(spec.slots):
+        for which, names in slots_.items():
+            put(i, which, names, axis=1 if (which == hm.HW_OUT_PROJ and len(names) > 1) else 0)
+    m.alloc_cache(-(-max_tokens // 64))
+    return m, nbytes
+
+
+def time_calls(call, sync, reps=5, settle_ms=200.0):
+    t, n = 0.0, 0
+    while t < settle_ms and n < 20:
+        t0 = time.perf_counter(); call(); sync(); t += (time.perf_counter() - t0) * 1e3; n += 1
+    d = []
+    for _ in range(reps):
+        sync(); t0 = time.perf_counter(); call(); sync(); d.append(time.perf_counter() - t0)
+    return sorted(d)[len(d) // 2]
+
+
+def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16):
+    import torch
+    from candle_vllm_amd import dense_model as DM
+    from candle_vllm_amd.block_engine import BlockEngine
+    from candle_vllm_amd.step_engine import StepEngine
+    from oracle.dense_llama import DenseConfig
+    s = SIZES[name]
+    cfg = sogodra_config(s)
+    rng = np.random.default_rng(5)
+    out = {"size": name, "shape": s, "prompt_tokens": T, "decode_batch": B, "decode_ctx": ctx}
+    sync = torch.cuda.synchronize
+    # ---- hybrid: prompt step, then B sequences decoding behind ctx tokens
+    hyb, wbytes = build_hybrid(cfg, max(T, B * (ctx + 1024)) + 64, slots=max(4, B))
+    eng = StepEngine(hyb, max(T, B * (ctx + 1024)) + 64)
+    toks = rng.integers(0, s["vocab"], T).tolist()
+
+    def prompt_h():
+        eng.feed("p", toks)
+        eng.step(["p"])
+        eng.finish("p")
+    dt = time_calls(prompt_h, sync, reps=3)
+    out["hybrid_prompt_tok_s"] = round(T / dt, 1)
+    ids = ["s%d" % i for i in range(B)]
+    for r in ids:
+        eng.feed(r, rng.integers(0, s["vocab"], ctx).tolist())
+        eng.step([r])
+
+    def decode_h():
+        for _ in range(dec_steps):
+            for r in ids:
+                eng.feed(r, [1])
+            eng.step(ids)
+    dt = time_calls(decode_h, sync, reps=3)
+    out["hybrid_decode_tok_s"] = round(B * dec_steps / dt, 1)
+    out["hybrid_decode_ms_per_step"] = round(dt / dec_steps * 1e3, 3)
+    out["hybrid_weight_GB"] = round(wbytes / 1e9, 3)
+    out["hybrid_decode_weight_GBs"] = round(wbytes * dec_steps / dt / 1e9, 1)
+    del eng, hyb
+    torch.cuda.empty_cache()
+    # ---- the llama host layer at equal size
+    n_layers = len(s["layers"])
+    dc = DenseConfig(hidden=s["width"], n_layers=n_layers, n_heads=s["heads"], n_kv_heads=s["kv"], head_dim=s["dim"], intermediate=s["ff"],
+                     vocab=s["vocab"], max_seq=8192, block_size=64)
+    nblk = B * (-(-(ctx + 64) // 64)) + (-(-T // 64)) + 2
+    gm = DM.DenseLlama(dc, max_batch=B, max_blocks_per_seq=-(-max(T, ctx + 64) // 64) + 1, kv_layout=DM.KV_PAGED)
+    gm.load_synthetic()
+    gm.alloc_kv_cache(nblk)
+    be = BlockEngine(64, nblk, 0)
+    seq = be.new_sequence(1000, toks)
+    be.allocate([seq], chunk=T)
+    meta = be.prepare_prompt([seq])
+    dt = time_calls(lambda: gm.forward(meta, is_prefill=True, sync=False), sync, reps=3)
+    out["llama_prompt_tok_s"] = round(T / dt, 1)
+    be.free_sequence(seq)
+    seqs = []
+    for i in range(B):
+        q = be.new_sequence(i, rng.integers(0, s["vocab"], ctx + 1).tolist())
+        be.allocate([q], chunk=ctx + 64)
+        seqs.append(q)
+    dmeta = be.prepare_decode(seqs)
+
+    def decode_l():
+        for _ in range(dec_steps):
+            gm.forward(dmeta, is_prefill=False, sync=False)
+    dt = time_calls(decode_l, sync, reps=3)
+    out["llama_decode_tok_s"] = round(B * dec_steps / dt, 1)
+    out["llama_decode_ms_per_step"] = round(dt / dec_steps * 1e3, 3)
+    out["llama_weight_GB"] = round(gm.weight_bytes() / 1e9, 3)
+    out["llama_decode_weight_GBs"] = round(gm.weight_bytes() * dec_steps / dt / 1e9, 1)
+    out["prompt_ratio_hybrid_over_llama"] = round(out["hybrid_prompt_tok_s"] / out["llama_prompt_tok_s"], 3)
+    out["decode_ratio_hybrid_over_llama"] = round(out["hybrid_decode_tok_s"] / out["llama_decode_tok_s"], 3)
+    del gm
+    torch.cuda.empty_cache()
+    return out
+
+
+def main(sizes="1b,3b", prompt_tokens=2048, batch=8, ctx=2048):
+    res = [run_size(n.strip(), T=prompt_tokens, B=batch, ctx=ctx) for n in sizes.split(",") if n.strip()]
+    print(json.dumps({"metric": "hybrid_vs_llama_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
+                      "note": "Sogodra layer-list host layer beside the 16-bit llama host layer at equal sizes; eager steps", "sizes": res}))

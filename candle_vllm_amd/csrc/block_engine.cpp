@@ -1049,6 +1049,11 @@ int32_t mi355_sched_schedule(void* sp, uint64_t now_ms) {
             size_t individual = 0;
             for (int64_t rg : s->running) individual += s->g(rg).seqs.size();
             if ((int)individual + 1 > s->max_parallel) break;
+            if (e->state_slots > 0) {                                              // stateful models: a group runs only with a state
+                int need = 0;                                                      // slot per sequence; a group between two chunks of
+                for (int64_t sid : gr.seqs) if (!e->state_of.count(sid)) ++need;   // its prompt keeps the one it has
+                if (need > (int)e->state_free.size()) break;
+            }
             if (!s->has_block_table(gr)) {
                 const int st = mi355_be_can_allocate(e, gr.seqs.data(), (int)gr.seqs.size(), s->chunk);
                 if (st == 1) break;                                                // Later
@@ -1062,6 +1067,7 @@ int32_t mi355_sched_schedule(void* sp, uint64_t now_ms) {
             } else if (!s->ensure_prefill_chunk_slots(gr)) {
                 break;
             }
+            if (e->state_slots > 0) for (int64_t sid : gr.seqs) (void)mi355_be_state_acquire(e, sid);
             gr.status = G_RUNNING;
             s->waiting.pop_front();
             s->running.push_back(gid);

@@ -31,13 +31,18 @@ def run_engine(gm, sched, requests, chunk=0, bt_width=None, ctx_cap=None, stream
     import torch
     from . import ops as cvo
     eng = sched.block_engine
-    bt_width = bt_width or int(gm.c.max_blocks_per_seq)
-    ctx_cap = ctx_cap or min(gm.cfg.max_seq, bt_width * gm.cfg.block_size)
+    stateful = bool(getattr(gm, "stateful", False))       # layers that carry state from token to token (hybrid_model.HybridModel):
+    if stateful:                                          # every running sequence holds a state slot of the block engine; prompt
+        graph = False                                     # portions and decoded tokens go through the model's one step function
+    else:
+        bt_width = bt_width or int(gm.c.max_blocks_per_seq)
+        ctx_cap = ctx_cap or min(gm.cfg.max_seq, bt_width * gm.cfg.block_size)
     pending = sorted(requests, key=lambda r: (r.arrival_step, r.id))
     by_id = {r.id: r for r in requests}
     done, step, pi = set(), 0, 0
     stats = dict(prompt_steps=0, decode_steps=0, prompt_tokens=0, max_batch=0, preempted=0, batch_hist={}, idle_steps=0)
-    gm.set_graph(bool(graph))
+    if not stateful:
+        gm.set_graph(bool(graph))
     t0 = time.perf_counter()
     while len(done) < len(requests) and step < max_steps:
         while pi < len(pending) and pending[pi].arrival_step <= step:
@@ -67,7 +72,7 @@ def run_engine(gm, sched, requests, chunk=0, bt_width=None, ctx_cap=None, stream
             continue
         if out.is_prompt:
             meta = eng.prepare_prompt(group, chunk=chunk)
-            logits = gm.forward_prefill(meta)
+            logits = gm.forward_prefill(meta, [eng.state_acquire(q) for q in group]) if stateful else gm.forward_prefill(meta)
             toks = cvo.argmax(logits).cpu().numpy()
             sampled = set(sched.filter_prefill_finished(out.scheduled)) if chunk else set(out.scheduled)
             rows = {row: logits[row].cpu().numpy() for row, gid in enumerate(out.scheduled) if gid in trace_ids}
@@ -76,6 +81,16 @@ def run_engine(gm, sched, requests, chunk=0, bt_width=None, ctx_cap=None, stream
         else:
             meta = eng.prepare_decode(group)
             B = len(group)
+            if stateful:                                               # a decoded token = a portion of one token behind its context
+                meta["cu_seqlens_q"] = np.arange(B + 1, dtype=np.uint32)
+                logits = gm.step(meta, [eng.state_acquire(q) for q in group])
+                toks = cvo.argmax(logits).cpu().numpy()
+                rows = {row: logits[row].cpu().numpy() for row, gid in enumerate(out.scheduled) if gid in trace_ids}
+                sampled = set(out.scheduled)
+                stats["decode_steps"] += 1
+                stats["max_batch"] = max(stats["max_batch"], B)
+                stats["batch_hist"][B] = stats["batch_hist"].get(B, 0) + 1
+        if not out.is_prompt and not stateful:
             bt = np.zeros((B, bt_width), np.uint32)
             w = meta["block_tables"].shape[1]
             bt[:, :w] = meta["block_tables"]
