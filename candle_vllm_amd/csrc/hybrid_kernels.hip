@@ -109,6 +109,82 @@ template <typename TA, int MT> __global__ __launch_bounds__(256) void linear_bf1
         }
 }
 
+// Prompt-sized products whose operands are both bf16 with 16-byte aligned rows and K a multiple of 32: a workgroup of four waves
+// owns a 128-token x 128-column tile, each wave a 64 x 64 quarter (4 x 4 MFMA tiles).  The 128 x 32 slices of both operands go
+// through LDS (rows padded to 80 bytes so that the 16 rows a fragment read touches fall into different 16-byte banks), the slice
+// of the next K step is fetched into registers while the current one is multiplied: one barrier per K step.
+__global__ __launch_bounds__(256) void linear_bf16_lds_kernel(LinArgs p) {
+    constexpr int ROWB = 80;                                        // bytes per staged row: 64 of data + 16 of padding
+    __shared__ __align__(16) uint8_t sa[2][128 * ROWB], sw[2][128 * ROWB];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, m16 = lane & 15, kg = lane >> 4;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int n0 = blockIdx.x * 128, t0 = blockIdx.y * 128;
+    const uint16_t* A = static_cast<const uint16_t*>(p.a);
+    const uint16_t* W = static_cast<const uint16_t*>(p.w);
+    // staging: thread -> rows r0 and r0 + 64 of both slices, 16-byte chunk ch of the 64-byte row
+    const int r0 = tid >> 2, ch = tid & 3;
+    const uint16_t* asrc[2]; const uint16_t* wsrc[2]; bool aok[2], wok[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int t = t0 + r0 + 64 * j, n = n0 + r0 + 64 * j;
+        aok[j] = t < p.T; wok[j] = n < p.N;
+        asrc[j] = A + (size_t)(aok[j] ? t : 0) * p.lda + ch * 8;
+        wsrc[j] = W + (size_t)(wok[j] ? n : 0) * p.K + ch * 8;
+    }
+    uint4 ra[2], rw[2];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            ra[j] = aok[j] ? *reinterpret_cast<const uint4*>(asrc[j] + k0) : uint4{0, 0, 0, 0};
+            rw[j] = wok[j] ? *reinterpret_cast<const uint4*>(wsrc[j] + k0) : uint4{0, 0, 0, 0};
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            *reinterpret_cast<uint4*>(&sa[buf][(r0 + 64 * j) * ROWB + ch * 16]) = ra[j];
+            *reinterpret_cast<uint4*>(&sw[buf][(r0 + 64 * j) * ROWB + ch * 16]) = rw[j];
+        }
+    };
+    f32x4_t acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    fetch(0);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    for (int k0 = 0; k0 < p.K; k0 += 32, buf ^= 1) {
+        const bool more = k0 + 32 < p.K;
+        if (more) fetch(k0 + 32);
+        uint4 af[4], bf[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) af[i] = *reinterpret_cast<const uint4*>(&sa[buf][(wr * 64 + i * 16 + m16) * ROWB + kg * 16]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) bf[j] = *reinterpret_cast<const uint4*>(&sw[buf][(wc * 64 + j * 16 + m16) * ROWB + kg * 16]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[i][j] = mfma_bf16(af[i], bf[j], acc[i][j]);
+        if (more) stage(buf ^ 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int n = n0 + wc * 64 + j * 16 + m16;
+        if (n >= p.N) continue;
+        const float bias = p.bias ? p.bias[n] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int t = t0 + wr * 64 + i * 16 + 4 * kg + v;
+                if (t < p.T) p.out[(size_t)t * p.ldo + n] = acc[i][j][v] + bias;
+            }
+    }
+}
+
 // Up to 16 tokens, bf16 weights: the product is a stream over the weights.  A workgroup owns 16 weight rows; its NW waves take the
 // 32-wide K steps in turn (UNR steps in flight per wave) and add their partial tiles through LDS.
 template <typename TA, int NW, int UNR> __global__ __launch_bounds__(64 * NW) void linear_bf16_stream_kernel(LinArgs p) {
@@ -302,16 +378,37 @@ struct AttnArgs {
     void* out; int ldo, out_off;
     const void* q; const void* k_pages; const void* v_pages;
     const uint32_t* bt; const uint32_t* ctx; const uint32_t* cu_q; const int32_t* tok_seq; const float* sink;
-    int n_seqs, H, G, d, vd, bs, max_blocks, window; float scale, out_scale;
+    int n_seqs, H, G, d, vd, bs, max_blocks, window; float scale, out_scale; int cp2;
 };
+// 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
+template <typename TC> struct Vec16;
+template <> struct Vec16<uint16_t> {
+    static constexpr int N = 8;
+    static __device__ __forceinline__ void load(const uint16_t* p, float* x) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        x[0] = bf16lo_to_f32(v.x); x[1] = bf16hi_to_f32(v.x); x[2] = bf16lo_to_f32(v.y); x[3] = bf16hi_to_f32(v.y);
+        x[4] = bf16lo_to_f32(v.z); x[5] = bf16hi_to_f32(v.z); x[6] = bf16lo_to_f32(v.w); x[7] = bf16hi_to_f32(v.w);
+    }
+};
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    static __device__ __forceinline__ void load(const float* p, float* x) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        x[0] = v.x; x[1] = v.y; x[2] = v.z; x[3] = v.w;
+    }
+};
+
 // One workgroup of NW waves per (new token, head).  Wave w takes the 64-key chunks w, w + NW, ... of the token's window: a lane
-// scores one key (q from LDS, the key row from its page), the wave keeps a running maximum / denominator / value sum (vd / 64
-// columns per lane), and the waves' partial results are merged through LDS.  The sink enters as a partial result with maximum
-// sink, denominator 1 and no value.
-template <typename TC, typename TO, int NW, int VPL> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
-    extern __shared__ float smem[];
-    float* qs = smem;                                   // [d]
-    float* pm = qs + p.d;                               // [NW] maxima, [NW] denominators, [NW][vd] sums
+// scores one key (q from LDS, the key row from its page), the wave keeps a running maximum / denominator / value sum, and the waves'
+// partial results are merged through LDS.  The sink enters the merge as a partial result with maximum sink, denominator 1 and no
+// value.  VEC (head sizes that are multiples of 16 bytes): rows are read 16 bytes at a time; for the value sum the wave's lanes
+// are (key, 16-byte chunk of the row) pairs -- 64 / cp2 keys per pass -- and the keys' partial sums are added by lane exchanges.
+template <typename TC, typename TO, int NW, bool VEC> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
+    constexpr int EPV = Vec16<TC>::N;
+    constexpr int NACC = VEC ? EPV : 8;
+    extern __shared__ __align__(16) float smem[];
+    float* qs = smem;                                   // [d rounded up to 4]
+    float* pm = qs + ((p.d + 3) & ~3);                  // [NW] maxima, [NW] denominators, [NW][vd] sums
     float* pl = pm + NW;
     float* pacc = pl + NW;
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -324,9 +421,11 @@ template <typename TC, typename TO, int NW, int VPL> __global__ __launch_bounds_
     for (int i = threadIdx.x; i < p.d; i += blockDim.x) qs[i] = ld<TC>(q, i);
     __syncthreads();
     const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
-    float m = -INFINITY, l = 0.f, acc[VPL];
+    const int cp2 = p.cp2, chunk = lane & (cp2 - 1), ksub = lane / cp2, kpp = 64 / cp2;     // VEC only
+    const bool chunk_ok = chunk * EPV < p.vd;
+    float m = -INFINITY, l = 0.f, acc[NACC];
 #pragma unroll
-    for (int e = 0; e < VPL; ++e) acc[e] = 0.f;
+    for (int e = 0; e < NACC; ++e) acc[e] = 0.f;
     for (int j0 = lo + wave * 64; j0 <= pos; j0 += NW * 64) {
         const int j = j0 + lane;
         float sc = -INFINITY;
@@ -335,7 +434,16 @@ template <typename TC, typename TO, int NW, int VPL> __global__ __launch_bounds_
             page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
             const TC* kr = static_cast<const TC*>(p.k_pages) + ((size_t)page_row * p.G + g) * p.d;
             float dot = 0.f;
-            for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
+            if (VEC) {
+                for (int i = 0; i < p.d; i += EPV) {
+                    float x[EPV];
+                    Vec16<TC>::load(kr + i, x);
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) dot = fmaf(qs[i + e], x[e], dot);
+                }
+            } else {
+                for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
+            }
             sc = dot * p.scale;
         }
         const float mn = fmaxf(m, wave_max(sc));
@@ -343,38 +451,56 @@ template <typename TC, typename TO, int NW, int VPL> __global__ __launch_bounds_
         const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
         l = l * corr + wave_sum(pj);
 #pragma unroll
-        for (int e = 0; e < VPL; ++e) acc[e] *= corr;
+        for (int e = 0; e < NACC; ++e) acc[e] *= corr;
         m = mn;
         const int cnt = min(64, pos - j0 + 1);
-        for (int jj = 0; jj < cnt; ++jj) {
-            const float pv = __shfl(pj, jj);
-            const size_t pr = (size_t)__shfl(page_row, jj);
-            const TC* vr = static_cast<const TC*>(p.v_pages) + (pr * p.G + g) * p.vd;
+        if (VEC) {
+            for (int k0 = 0; k0 < cnt; k0 += kpp) {
+                const int jj = k0 + ksub;
+                const float pv = __shfl(pj, jj & 63);
+                const size_t pr = (size_t)__shfl(page_row, jj & 63);
+                if (jj < cnt && chunk_ok) {
+                    float x[EPV];
+                    Vec16<TC>::load(static_cast<const TC*>(p.v_pages) + (pr * p.G + g) * p.vd + chunk * EPV, x);
 #pragma unroll
-            for (int e = 0; e < VPL; ++e) { const int c = lane + 64 * e; if (c < p.vd) acc[e] = fmaf(pv, ld<TC>(vr, c), acc[e]); }
+                    for (int e = 0; e < EPV; ++e) acc[e] = fmaf(pv, x[e], acc[e]);
+                }
+            }
+        } else {
+            for (int jj = 0; jj < cnt; ++jj) {
+                const float pv = __shfl(pj, jj);
+                const size_t pr = (size_t)__shfl(page_row, jj);
+                const TC* vr = static_cast<const TC*>(p.v_pages) + (pr * p.G + g) * p.vd;
+#pragma unroll
+                for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) acc[e] = fmaf(pv, ld<TC>(vr, c), acc[e]); }
+            }
         }
     }
     if (lane == 0) { pm[wave] = m; pl[wave] = l; }
+    if (VEC) {
+        for (int off = cp2; off < 64; off <<= 1)
 #pragma unroll
-    for (int e = 0; e < VPL; ++e) { const int c = lane + 64 * e; if (c < p.vd) pacc[wave * p.vd + c] = acc[e]; }
+            for (int e = 0; e < NACC; ++e) acc[e] += __shfl_xor(acc[e], off);
+        if (ksub == 0 && chunk_ok)
+#pragma unroll
+            for (int e = 0; e < EPV; ++e) pacc[wave * p.vd + chunk * EPV + e] = acc[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) pacc[wave * p.vd + c] = acc[e]; }
+    }
     __syncthreads();
     if (wave == 0) {
         float M = p.sink ? p.sink[h] : -INFINITY;
         for (int w = 0; w < NW; ++w) M = fmaxf(M, pm[w]);
         float L = p.sink ? expf(p.sink[h] - M) : 0.f;
-        float o[VPL];
-#pragma unroll
-        for (int e = 0; e < VPL; ++e) o[e] = 0.f;
-        for (int w = 0; w < NW; ++w) {
-            if (pm[w] == -INFINITY) continue;
-            const float c = expf(pm[w] - M);
-            L += pl[w] * c;
-#pragma unroll
-            for (int e = 0; e < VPL; ++e) { const int col = lane + 64 * e; if (col < p.vd) o[e] += pacc[w * p.vd + col] * c; }
-        }
+        float cw[NW];
+        for (int w = 0; w < NW; ++w) { cw[w] = pm[w] == -INFINITY ? 0.f : expf(pm[w] - M); L += pl[w] * cw[w]; }
         TO* out = static_cast<TO*>(p.out) + (size_t)t * p.ldo + p.out_off + (size_t)h * p.vd;
-#pragma unroll
-        for (int e = 0; e < VPL; ++e) { const int col = lane + 64 * e; if (col < p.vd) st<TO>(out, col, o[e] / L * p.out_scale); }
+        for (int col = lane; col < p.vd; col += 64) {
+            float o = 0.f;
+            for (int w = 0; w < NW; ++w) o += pacc[w * p.vd + col] * cw[w];
+            st<TO>(out, col, o / L * p.out_scale);
+        }
     }
 }
 
@@ -435,78 +561,127 @@ struct DeltaArgs {
     const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots;
     int H, G, d, vd; float unit_eps;
 };
-// One workgroup per (sequence, head); thread j owns column j of the state S [d, vd] in registers and walks the new tokens in order:
+// Everything of the rule that does not depend on the state is computed for all new tokens at once, one wave per (token, head):
+// prep [T, P] = unit q times d^-1/2 and unit k per q/k head, the decays per head (or per head and key channel), beta per head.
+__global__ __launch_bounds__(64) void delta_prep_kernel(DeltaArgs p, float* prep, int P, int T) {
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const int d = p.d, hpg = p.H / p.G, g = h / hpg;
+    float* out = prep + (size_t)t * P;
+    const int q_off = 0, k_off = p.G * d, g_off = 2 * p.G * d, dd = p.decay_channels ? d : 1, b_off = g_off + p.H * dd;
+    if (h % hpg == 0) {
+        const float* row = p.qkv + (size_t)t * p.ldq;
+        float qq = 0.f, kk = 0.f;
+        for (int i = lane; i < d; i += 64) { const float a = row[g * d + i], b = row[p.G * d + g * d + i]; qq += a * a; kk += b * b; }
+        qq = wave_sum(qq); kk = wave_sum(kk);
+        const float qi = (1.f / sqrtf((float)d)) / sqrtf(qq + p.unit_eps), ki = 1.f / sqrtf(kk + p.unit_eps);
+        for (int i = lane; i < d; i += 64) {
+            out[q_off + g * d + i] = row[g * d + i] * qi;
+            out[k_off + g * d + i] = row[p.G * d + g * d + i] * ki;
+        }
+    }
+    const float a_rate = expf(p.a_log[h]);
+    if (p.decay_channels) {
+        for (int i = lane; i < d; i += 64) {
+            const int ch = h * d + i;
+            out[g_off + ch] = expf(-a_rate * softplusf_(p.decay_in[(size_t)t * p.ldd + ch] + p.dt_bias[ch]));
+        }
+    } else if (lane == 0) {
+        out[g_off + h] = expf(-a_rate * softplusf_(p.decay_in[(size_t)t * p.ldd + h] + p.dt_bias[h]));
+    }
+    if (lane == 0) out[b_off + h] = sigmoidf_(p.proj[(size_t)t * p.ldp + p.b_off + h]);
+}
+
+// The scan.  A workgroup of 256 threads owns 64 columns of one (sequence, head)'s state S [d, vd]; four neighbouring lanes share a
+// column, each holding DP = ceil(d / 4) of its rows in registers, and walk the new tokens in order:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
-// CH tokens at a time are staged in LDS: unit q (times d^-1/2), unit k, the decays and beta, computed by the whole workgroup.
-template <int D, int CH> __global__ __launch_bounds__(256) void delta_rule_kernel(DeltaArgs p) {
-    __shared__ float sq[CH][D], sk[CH][D], sg[CH][D];
-    __shared__ float sbeta[CH], sgh[CH];
-    const int s = blockIdx.x, h = blockIdx.y, nt = blockDim.x;
-    const int tid = blockIdx.z * nt + threadIdx.x;                  // the state column; a workgroup holds up to 256 of them
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = nt >> 6;
-    const int g = h / (p.H / p.G);
+// (the two sums over d are finished by two lane exchanges inside the quad).  q, k, g of CH tokens at a time sit in LDS, rows padded
+// so that the four parts fall into different banks; the next CH tokens are fetched into registers while the current ones are used.
+template <int DP, int CH> __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs p, const float* __restrict__ prep, int P) {
+    constexpr int RS = DP + 4, TOT = CH * 4 * DP, NPT = (TOT + 255) / 256;
+    __shared__ __align__(16) float sq[2][CH][4][RS], sk[2][CH][4][RS], sg[2][CH][4][RS];
+    __shared__ float sb[2][CH], sgh[2][CH];
+    const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+    const int col = blockIdx.z * 64 + (tid >> 2), part = tid & 3;
+    const int d = p.d, vd = p.vd, g = h / (p.H / p.G);
     const int tb = (int)p.cu_q[s], te = (int)p.cu_q[s + 1];
     if (te <= tb) return;
     const int start_pos = (int)p.ctx[s] - (te - tb);
-    const int d = p.d, vd = p.vd;
-    const bool own = tid < vd;
+    const bool own = col < vd, chan = p.decay_channels != 0;
     float* stt = p.state + (size_t)p.slots[s] * p.state_stride + (size_t)h * d * vd;
-    float S[D];
+    float S[DP];
 #pragma unroll
-    for (int i = 0; i < D; ++i) S[i] = (own && i < d && start_pos > 0) ? stt[(size_t)i * vd + tid] : 0.f;
-    const int q_col = g * d, k_col = p.G * d + g * d, v_col = 2 * p.G * d + h * vd;
-    const float a_rate = expf(p.a_log[h]);
-    const float q_scale = 1.f / sqrtf((float)d);
-    for (int t0 = tb; t0 < te; t0 += CH) {
-        const int cn = min(CH, te - t0);
-        __syncthreads();
-        // unit vectors: wave w normalises the q and k of tokens w, w + nw, ...
-        for (int c = wave; c < cn; c += nw) {
-            const float* row = p.qkv + (size_t)(t0 + c) * p.ldq;
-            float qq = 0.f, kk = 0.f;
-            for (int i = lane; i < d; i += 64) { const float a = row[q_col + i], b = row[k_col + i]; qq += a * a; kk += b * b; }
-            qq = wave_sum(qq); kk = wave_sum(kk);
-            const float qi = q_scale / sqrtf(qq + p.unit_eps), ki = 1.f / sqrtf(kk + p.unit_eps);
-            for (int i = lane; i < D; i += 64) {
-                sq[c][i] = i < d ? row[q_col + i] * qi : 0.f;
-                sk[c][i] = i < d ? row[k_col + i] * ki : 0.f;
-                if (p.decay_channels) {
-                    const int ch = h * d + i;
-                    sg[c][i] = i < d ? expf(-a_rate * softplusf_(p.decay_in[(size_t)(t0 + c) * p.ldd + ch] + p.dt_bias[ch])) : 1.f;
-                }
-            }
-            if (lane == 0) {
-                sbeta[c] = sigmoidf_(p.proj[(size_t)(t0 + c) * p.ldp + p.b_off + h]);
-                if (!p.decay_channels) sgh[c] = expf(-a_rate * softplusf_(p.decay_in[(size_t)(t0 + c) * p.ldd + h] + p.dt_bias[h]));
+    for (int r = 0; r < DP; ++r) { const int i = part * DP + r; S[r] = (own && i < d && start_pos > 0) ? stt[(size_t)i * vd + col] : 0.f; }
+    const int q_off = g * d, k_off = p.G * d + g * d, g_off = 2 * p.G * d + (chan ? h * d : h), b_off = 2 * p.G * d + p.H * (chan ? d : 1) + h;
+    const int v_col = 2 * p.G * d + h * vd + col;
+    float rq[NPT], rk[NPT], rg[NPT], rv[CH], rbeta = 0.f, rgh = 1.f;
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int n = 0; n < NPT; ++n) {
+            const int idx = tid + n * 256, c = idx / (4 * DP), ii = idx - c * (4 * DP), t = t0 + c;
+            const bool ok_ = idx < TOT && t < te && ii < d;
+            const float* row = prep + (size_t)(ok_ ? t : tb) * P;
+            rq[n] = ok_ ? row[q_off + ii] : 0.f;
+            rk[n] = ok_ ? row[k_off + ii] : 0.f;
+            rg[n] = (ok_ && chan) ? row[g_off + ii] : 1.f;
+        }
+#pragma unroll
+        for (int c = 0; c < CH; ++c) rv[c] = (own && t0 + c < te) ? p.qkv[(size_t)(t0 + c) * p.ldq + v_col] : 0.f;
+        if (tid < CH && t0 + tid < te) {
+            rbeta = prep[(size_t)(t0 + tid) * P + b_off];
+            rgh = chan ? 1.f : prep[(size_t)(t0 + tid) * P + g_off];
+        }
+    };
+    auto stage = [&](int buf) {
+#pragma unroll
+        for (int n = 0; n < NPT; ++n) {
+            const int idx = tid + n * 256;
+            if (idx < TOT) {
+                const int c = idx / (4 * DP), ii = idx - c * (4 * DP), pp = ii / DP, r = ii - pp * DP;
+                sq[buf][c][pp][r] = rq[n]; sk[buf][c][pp][r] = rk[n]; sg[buf][c][pp][r] = rg[n];
             }
         }
-        float vv[CH];
+        if (tid < CH) { sb[buf][tid] = rbeta; sgh[buf][tid] = rgh; }
+    };
+    fetch(tb);
+    stage(0);
+    __syncthreads();
+    int buf = 0;
+    for (int t0 = tb; t0 < te; t0 += CH, buf ^= 1) {
+        float vc[CH];
 #pragma unroll
-        for (int c = 0; c < CH; ++c) vv[c] = (own && c < cn) ? p.qkv[(size_t)(t0 + c) * p.ldq + v_col + tid] : 0.f;
-        __syncthreads();
-        if (own) {
-#pragma unroll 1
-            for (int c = 0; c < cn; ++c) {
+        for (int c = 0; c < CH; ++c) vc[c] = rv[c];
+        const bool more = t0 + CH < te;
+        if (more) fetch(t0 + CH);
+        const int cn = min(CH, te - t0);
+#pragma unroll
+        for (int c = 0; c < CH; ++c) {
+            if (c < cn) {
                 float kv = 0.f;
-                if (p.decay_channels) {
+                if (chan) {
 #pragma unroll
-                    for (int i = 0; i < D; ++i) { S[i] *= sg[c][i]; kv = fmaf(S[i], sk[c][i], kv); }
+                    for (int r = 0; r < DP; ++r) { S[r] *= sg[buf][c][part][r]; kv = fmaf(S[r], sk[buf][c][part][r], kv); }
                 } else {
-                    const float gh = sgh[c];
+                    const float gh = sgh[buf][c];
 #pragma unroll
-                    for (int i = 0; i < D; ++i) { S[i] *= gh; kv = fmaf(S[i], sk[c][i], kv); }
+                    for (int r = 0; r < DP; ++r) { S[r] *= gh; kv = fmaf(S[r], sk[buf][c][part][r], kv); }
                 }
-                const float u = sbeta[c] * (vv[c] - kv);
+                kv += __shfl_xor(kv, 1);
+                kv += __shfl_xor(kv, 2);
+                const float u = sb[buf][c] * (vc[c] - kv);
                 float o = 0.f;
 #pragma unroll
-                for (int i = 0; i < D; ++i) { S[i] = fmaf(sk[c][i], u, S[i]); o = fmaf(S[i], sq[c][i], o); }
-                p.o[((size_t)(t0 + c) * p.H + h) * vd + tid] = o;
+                for (int r = 0; r < DP; ++r) { S[r] = fmaf(sk[buf][c][part][r], u, S[r]); o = fmaf(S[r], sq[buf][c][part][r], o); }
+                o += __shfl_xor(o, 1);
+                o += __shfl_xor(o, 2);
+                if (own && part == 0) p.o[((size_t)(t0 + c) * p.H + h) * vd + col] = o;
             }
         }
+        if (more) stage(buf ^ 1);
+        __syncthreads();
     }
     if (own)
 #pragma unroll
-        for (int i = 0; i < D; ++i) if (i < d) stt[(size_t)i * vd + tid] = S[i];
+        for (int r = 0; r < DP; ++r) { const int i = part * DP + r; if (i < d) stt[(size_t)i * vd + col] = S[r]; }
 }
 
 // out = o / rms(o) * w * gate * out_scale, one wave per (token, head)
@@ -625,6 +800,8 @@ int mi355_hyb_linear(float* out, int32_t ldo, const void* a, int32_t a_dtype, in
         const dim3 grid((n + 15) / 16);
         if (k >= 2048) { if (af) linear_bf16_stream_kernel<float, 4, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 4, 4><<<grid, 256, 0, st_>>>(p); }
         else { if (af) linear_bf16_stream_kernel<float, 2, 2><<<grid, 128, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 2, 2><<<grid, 128, 0, st_>>>(p); }
+    } else if (T > 32 && !af && p.a_vec && p.w_vec && k % 32 == 0) {
+        linear_bf16_lds_kernel<<<dim3((n + 127) / 128, (T + 127) / 128), 256, 0, st_>>>(p);
     } else if (T <= 32) {
         const dim3 grid((n + 63) / 64, (T + 31) / 32);
         if (af) linear_bf16_tile_kernel<float, 2><<<grid, 256, 0, st_>>>(p); else linear_bf16_tile_kernel<uint16_t, 2><<<grid, 256, 0, st_>>>(p);
@@ -693,20 +870,23 @@ int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
                                    int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
                                    int32_t max_blocks, int32_t window, float scale, float out_scale, int32_t dtype, int64_t stream) {
     if (!out || !q || !k_pages || !v_pages || !block_tables || !context_lens || !cu_seqlens_q || !tok_seq) return -1;
-    if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || vdim > 512) return -1;
+    if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return -1;
     if (block_size <= 0 || max_blocks <= 0 || window < 0) return -1;
     if (T <= 0) return 0;
     AttnArgs p{out, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq, sink,
-               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale};
+               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale, 64};
     constexpr int NW = 4;
-    const size_t lds = (size_t)(dim + 2 * NW + NW * vdim) * sizeof(float);
+    const size_t lds = (size_t)(((dim + 3) & ~3) + 2 * NW + NW * vdim) * sizeof(float);
     const dim3 grid(T, heads);
     hipStream_t s_ = to_stream(stream);
     const bool f = dtype == MI355_DTYPE_F32, of = out_dtype == MI355_DTYPE_F32;
-#define WA(TC, TO, VPL) window_attention_kernel<TC, TO, NW, VPL><<<grid, 64 * NW, lds, s_>>>(p)
-#define WA_V(TC, TO) do { if (vdim <= 64) WA(TC, TO, 1); else if (vdim <= 128) WA(TC, TO, 2); else if (vdim <= 256) WA(TC, TO, 4); else WA(TC, TO, 8); } while (0)
-    if (f && of) WA_V(float, float); else if (f) WA_V(float, uint16_t); else if (of) WA_V(uint16_t, float); else WA_V(uint16_t, uint16_t);
-#undef WA_V
+    const int epv = f ? 4 : 8;
+    const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0;
+    if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; }
+    else if (vdim > 512) return -1;
+#define WA(TC, TO) do { if (vec) window_attention_kernel<TC, TO, NW, true><<<grid, 64 * NW, lds, s_>>>(p); \
+                        else window_attention_kernel<TC, TO, NW, false><<<grid, 64 * NW, lds, s_>>>(p); } while (0)
+    if (f && of) WA(float, float); else if (f) WA(float, uint16_t); else if (of) WA(uint16_t, float); else WA(uint16_t, uint16_t);
 #undef WA
     LAUNCH_OK(); return 0;
 }
@@ -735,23 +915,31 @@ int mi355_hyb_conv_state_update(float* conv_state, int64_t state_stride, const f
     LAUNCH_OK(); return 0;
 }
 
+int mi355_hyb_delta_rule_scratch_floats(int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t decay_channels) {
+    return num_tokens * (2 * kv_heads * dim + heads * (decay_channels ? dim : 1) + heads);
+}
+
 int mi355_hyb_delta_rule(float* o, float* state, int64_t state_stride, const float* qkv, int32_t ldq, const float* proj, int32_t ldp,
                          int32_t b_off, const float* decay_in, int32_t ldd, int32_t decay_channels, const float* a_log,
                          const float* dt_bias, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
-                         int32_t num_seqs, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float unit_eps, int64_t stream) {
-    if (!o || !state || !qkv || !proj || !decay_in || !a_log || !dt_bias || !context_lens || !cu_seqlens_q || !state_slots) return -1;
+                         int32_t num_seqs, int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, float unit_eps,
+                         float* scratch, int64_t stream) {
+    if (!o || !state || !qkv || !proj || !decay_in || !a_log || !dt_bias || !context_lens || !cu_seqlens_q || !state_slots || !scratch) return -1;
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || dim > 256 || vdim <= 0) return -1;
-    if (num_seqs <= 0) return 0;
+    if (num_seqs <= 0 || num_tokens <= 0) return 0;
     DeltaArgs p{o, state, state_stride, qkv, ldq, proj, ldp, b_off, decay_in, ldd, decay_channels, a_log, dt_bias,
                 context_lens, cu_seqlens_q, state_slots, heads, kv_heads, dim, vdim, unit_eps};
-    const int threads = vdim >= 256 ? 256 : ((vdim + 63) / 64) * 64;
-    const dim3 grid(num_seqs, heads, (vdim + threads - 1) / threads);
     hipStream_t s_ = to_stream(stream);
-    if (dim <= 16) delta_rule_kernel<16, 8><<<grid, threads, 0, s_>>>(p);
-    else if (dim <= 32) delta_rule_kernel<32, 8><<<grid, threads, 0, s_>>>(p);
-    else if (dim <= 64) delta_rule_kernel<64, 8><<<grid, threads, 0, s_>>>(p);
-    else if (dim <= 128) delta_rule_kernel<128, 8><<<grid, threads, 0, s_>>>(p);
-    else delta_rule_kernel<256, 4><<<grid, threads, 0, s_>>>(p);
+    const int P = 2 * kv_heads * dim + heads * (decay_channels ? dim : 1) + heads;
+    delta_prep_kernel<<<dim3(num_tokens, heads), 64, 0, s_>>>(p, scratch, P, num_tokens);
+    LAUNCH_OK();
+    const dim3 grid(num_seqs, heads, (vdim + 63) / 64);
+    const int dp = (dim + 3) / 4;
+    if (dp <= 4) delta_scan_kernel<4, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+    else if (dp <= 8) delta_scan_kernel<8, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+    else if (dp <= 16) delta_scan_kernel<16, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+    else if (dp <= 32) delta_scan_kernel<32, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+    else delta_scan_kernel<64, 4><<<grid, 256, 0, s_>>>(p, scratch, P);
     LAUNCH_OK(); return 0;
 }
 

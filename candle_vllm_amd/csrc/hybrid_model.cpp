@@ -57,10 +57,10 @@ struct HModel {
     int num_blocks = 0;
     // activations (grow-only)
     int cap_t = 0, cap_out = 0;
-    float *x = nullptr, *proj = nullptr, *aux1 = nullptr, *aux2 = nullptr, *conv = nullptr, *o = nullptr, *y = nullptr, *gu = nullptr;
+    float *prep = nullptr, *x = nullptr, *proj = nullptr, *aux1 = nullptr, *aux2 = nullptr, *conv = nullptr, *o = nullptr, *y = nullptr, *gu = nullptr;
     void *xcopy = nullptr, *q = nullptr, *mix = nullptr, *act = nullptr, *xn = nullptr;
     int32_t* tok_seq = nullptr;
-    int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0;
+    int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0, max_prep = 0;
     bool bf16() const { return cfg.dtype == MI355_DTYPE_BF16; }
     size_t esize() const { return bf16() ? 2 : 4; }
 };
@@ -185,6 +185,7 @@ int ensure_capacity(HModel* m, int T, int n_out) {
         HCHECK(grow(m->aux2, t * (size_t)m->max_aux2 * 4));
         HCHECK(grow(m->conv, t * (size_t)m->max_conv * 4));
         HCHECK(grow(m->o, t * (size_t)m->max_o * 4));
+        HCHECK(grow(m->prep, t * (size_t)m->max_prep * 4));
         HCHECK(grow(m->y, t * W * 4));
         HCHECK(grow(m->gu, t * (size_t)m->max_ff * 2 * 4));
         HCHECK(grow(m->xcopy, t * W * 2));
@@ -239,6 +240,7 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
             if (c.d_gate == MI355_HYB_GATE_SIGMOID_LR) m->max_aux2 = std::max(m->max_aux2, c.d_heads * c.d_vdim);
             m->max_conv = std::max(m->max_conv, L.conv_channels());
             m->max_o = std::max(m->max_o, c.d_heads * c.d_vdim);
+            m->max_prep = std::max(m->max_prep, 2 * c.d_kv_heads * c.d_dim + c.d_heads * (c.d_decay_channels ? c.d_dim : 1) + c.d_heads);
             L.conv_off = off; off += (int64_t)L.conv_channels() * (c.d_conv - 1);
             L.state_off = off; off += (int64_t)c.d_heads * c.d_dim * c.d_vdim;
         }
@@ -257,7 +259,7 @@ void mi355_hybrid_destroy(void* mp) {
         for (Weight& w : L.w) if (w.p) (void)hipFree(w.p);
         for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.k_pages, L.v_pages}) if (p) (void)hipFree(p);
     }
-    for (void* p : {m->embed.p, m->final_norm.p, m->head.p, (void*)m->state, (void*)m->x, (void*)m->proj, (void*)m->aux1, (void*)m->aux2,
+    for (void* p : {m->embed.p, m->final_norm.p, m->head.p, (void*)m->state, (void*)m->prep, (void*)m->x, (void*)m->proj, (void*)m->aux1, (void*)m->aux2,
                     (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, (void*)m->tok_seq})
         if (p) (void)hipFree(p);
     delete m;
@@ -394,7 +396,7 @@ int mi355_hybrid_forward(void* mp, const uint32_t* tokens, const int64_t* positi
             }
             HCHECK(mi355_hyb_delta_rule(m->o, m->state + L.state_off, m->slot_floats, m->conv, C, m->proj, ldp, L.off[P_B], decay_in, ldd,
                                         c.d_decay_channels, f(MI355_HW_D_A_LOG), f(MI355_HW_D_DT_BIAS), context_lens, cu_seqlens_q,
-                                        state_slots, num_seqs, c.d_heads, c.d_kv_heads, c.d_dim, c.d_vdim, m->cfg.unit_eps, stream));
+                                        state_slots, num_seqs, T, c.d_heads, c.d_kv_heads, c.d_dim, c.d_vdim, m->cfg.unit_eps, m->prep, stream));
             HCHECK(mi355_hyb_gated_norm(m->mix, dt, L.out_k, mix_col, m->o, f(MI355_HW_D_NORM), gate_in, ldg, c.d_gate, T, c.d_heads,
                                         c.d_vdim, eps, c.mixer == MI355_HYB_MIX_PARALLEL ? c.d_out_scale : 1.f, stream));
         }

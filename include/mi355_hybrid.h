@@ -156,8 +156,10 @@ int mi355_hyb_conv_state_update(float* conv_state, int64_t state_stride, const f
 int mi355_hyb_delta_rule(float* o, float* state, int64_t state_stride, const float* qkv, int32_t ldq, const float* proj,
                          int32_t ldp, int32_t b_off, const float* decay_in, int32_t ldd, int32_t decay_channels,
                          const float* a_log, const float* dt_bias, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
-                         const int32_t* state_slots, int32_t num_seqs, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
-                         float unit_eps, int64_t stream);
+                         const int32_t* state_slots, int32_t num_seqs, int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim,
+                         int32_t vdim, float unit_eps, float* scratch, int64_t stream);
+/* floats of `scratch` (device): what the rule computes for all tokens at once before the scan over them */
+int mi355_hyb_delta_rule_scratch_floats(int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t decay_channels);
 /* out (dt_out) [T, ldo] at out_off = o / rms(o over vdim) * w * gate(gate_in) * out_scale; gate: MI355_HYB_GATE_* (silu / sigmoid) */
 int mi355_hyb_gated_norm(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const float* o, const float* w,
                          const float* gate_in, int32_t ldg, int32_t gate, int32_t num_tokens, int32_t heads, int32_t vdim, float eps,

@@ -261,10 +261,11 @@ def test_delta_rule_portions_and_state(lib, Hh, G, d, vd, per_channel):
     for lo, hi in ((0, 1), (1, 3), (3, 12), (12, 13), (13, 29)):
         n = hi - lo
         o = torch.zeros((n, Hh, vd), device="cuda")
+        scratch = torch.zeros(lib.mi355_hyb_delta_rule_scratch_floats(n, Hh, G, d, int(per_channel)), device="cuda")
         ok(lib.mi355_hyb_delta_rule(o.data_ptr(), state.data_ptr(), stride, P(qkv[lo:hi]), C, P(proj[lo:hi]), ldp,
                                     b_off, P(pre[lo:hi]), nd, int(per_channel), P(a_log), P(dtb),
-                                    P([hi], np.int32), P([0, n], np.int32), P([1], np.int32), 1, Hh, G,
-                                    d, vd, 1e-6, _st()))
+                                    P([hi], np.int32), P([0, n], np.int32), P([1], np.int32), 1, n, Hh, G,
+                                    d, vd, 1e-6, scratch.data_ptr(), _st()))
         got.append(o.cpu().numpy())
     got = np.concatenate(got)
     assert np.abs(got - want).max() < 2e-5 * max(1.0, np.abs(want).max())
