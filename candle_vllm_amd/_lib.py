@@ -366,6 +366,9 @@ _sig("mi355_hybrid_cache_bytes", c_i64, [c_vp, c_i32])
 _sig("mi355_hybrid_state_floats_per_slot", c_i64, [c_vp])
 _sig("mi355_hybrid_state_ptr", c_vp, [c_vp])
 _sig("mi355_hybrid_forward", ctypes.c_int, [c_vp] * 9 + [c_i32] * 5 + [c_vp, c_vp, c_i64])
+_sig("mi355_hybrid_forward_graph", ctypes.c_int, [c_vp] * 9 + [c_i32] * 5 + [c_vp, c_i64])
+_sig("mi355_hybrid_graph_captures", c_i64, [c_vp])
+_sig("mi355_hybrid_graph_replays", c_i64, [c_vp])
 _sig("mi355_hyb_token_seq", ctypes.c_int, [c_vp, c_vp, c_i32, c_i64])
 _sig("mi355_hyb_bf16_to_f32", ctypes.c_int, [c_vp, c_vp, c_i64, c_i64])
 _sig("mi355_hyb_copy_f32", ctypes.c_int, [c_vp, c_vp, c_i64, c_i64])

@@ -11,6 +11,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstring>
+#include <map>
 #include <vector>
 
 #include "../../include/mi355_hybrid.h"
@@ -61,9 +62,22 @@ struct HModel {
     void *xcopy = nullptr, *q = nullptr, *mix = nullptr, *act = nullptr, *xn = nullptr;
     int32_t* tok_seq = nullptr;
     int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0, max_prep = 0;
+    // captured steps (mi355_hybrid_forward_graph): one hipGraph per (device input pointers, counts); whatever re-allocates a buffer a
+    // step touches drops them all
+    struct StepGraph { hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; };
+    std::map<std::vector<int64_t>, StepGraph> graphs;
+    int64_t graph_captures = 0, graph_replays = 0;
     bool bf16() const { return cfg.dtype == MI355_DTYPE_BF16; }
     size_t esize() const { return bf16() ? 2 : 4; }
 };
+
+void drop_graphs(HModel* m) {
+    for (auto& kv : m->graphs) {
+        if (kv.second.exec) (void)hipGraphExecDestroy(kv.second.exec);
+        if (kv.second.graph) (void)hipGraphDestroy(kv.second.graph);
+    }
+    m->graphs.clear();
+}
 
 int in_proj_parts(const mi355_hybrid_layer& c, int32_t* off) {
     for (int i = 0; i < P_COUNT; ++i) off[i] = -1;
@@ -157,6 +171,7 @@ int store_weight(HModel* m, int layer, int which, const uint16_t* dev_bits, int6
     Weight* w = slot_of(m, layer, which);
     if (!w || n != expected_elems(m, layer, which)) return -2;
     const bool as_bf16 = is_matrix(which) && m->bf16();
+    drop_graphs(m);
     if (w->p) { (void)hipFree(w->p); w->p = nullptr; }
     HHIP(hipMalloc(&w->p, (size_t)n * (as_bf16 ? 2 : 4)));
     w->n = n;
@@ -179,6 +194,7 @@ int ensure_capacity(HModel* m, int T, int n_out) {
     if (T > m->cap_t) {
         const size_t t = (size_t)T, W = (size_t)m->cfg.width;
         HHIP(hipDeviceSynchronize());
+        drop_graphs(m);
         HCHECK(grow(m->x, t * W * 4));
         HCHECK(grow(m->proj, t * m->max_in_rows * 4));
         HCHECK(grow(m->aux1, t * (size_t)m->max_aux1 * 4));
@@ -197,6 +213,7 @@ int ensure_capacity(HModel* m, int T, int n_out) {
     }
     if (n_out > m->cap_out) {
         HHIP(hipDeviceSynchronize());
+        drop_graphs(m);
         HCHECK(grow(m->xn, (size_t)n_out * m->cfg.width * m->esize()));
         m->cap_out = n_out;
     }
@@ -255,6 +272,7 @@ void mi355_hybrid_destroy(void* mp) {
     HModel* m = static_cast<HModel*>(mp);
     if (!m) return;
     (void)hipDeviceSynchronize();
+    drop_graphs(m);
     for (HLayer& L : m->layers) {
         for (Weight& w : L.w) if (w.p) (void)hipFree(w.p);
         for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.k_pages, L.v_pages}) if (p) (void)hipFree(p);
@@ -289,6 +307,7 @@ int mi355_hybrid_set_rope_tables(void* mp, int32_t layer, const float* cos_t, co
     if (!m || layer < 0 || layer >= (int)m->layers.size() || !cos_t || !sin_t || n_positions <= 0) return -1;
     HLayer& L = m->layers[layer];
     if (!L.has_attn() || L.c.a_rot_dims <= 0) return -2;
+    drop_graphs(m);
     const size_t bytes = (size_t)n_positions * (L.c.a_rot_dims / 2) * 4;
     HHIP(hipDeviceSynchronize());
     HCHECK(grow(L.cos_t, bytes));
@@ -315,6 +334,7 @@ int mi355_hybrid_alloc_cache(void* mp, int32_t num_blocks) {
     HModel* m = static_cast<HModel*>(mp);
     if (!m || num_blocks <= 0) return -1;
     HHIP(hipDeviceSynchronize());
+    drop_graphs(m);
     for (HLayer& L : m->layers) {
         if (!L.has_attn()) continue;
         const size_t rows = (size_t)num_blocks * m->cfg.block_size * L.c.a_kv_heads;
@@ -331,11 +351,10 @@ int mi355_hybrid_alloc_cache(void* mp, int32_t num_blocks) {
     return 0;
 }
 
-int mi355_hybrid_forward(void* mp, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+static int forward_check(HModel* m, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
                          const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
                          const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t T,
-                         int32_t max_blocks, int32_t max_context_len, float* logits, float* layer_trace, int64_t stream) {
-    HModel* m = static_cast<HModel*>(mp);
+                         int32_t max_blocks, int32_t max_context_len, float* logits) {
     if (!m || !tokens || !positions || !slot_mapping || !block_tables || !context_lens || !cu_seqlens_q || !state_slots) return -1;
     if (num_seqs <= 0 || T <= 0 || n_out < 0 || (n_out > 0 && (!out_rows || !logits)) || max_blocks <= 0) return -1;
     if (!m->state || !m->embed.p || !m->final_norm.p || !m->head.p) return -3;
@@ -347,7 +366,13 @@ int mi355_hybrid_forward(void* mp, const uint32_t* tokens, const int64_t* positi
             if (s != MI355_HW_IN_BIAS && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
         if (L.has_attn() && (!L.k_pages || (L.c.a_rot_dims > 0 && L.n_pos < max_context_len))) return -4;
     }
-    HCHECK(ensure_capacity(m, T, n_out));
+    return ensure_capacity(m, T, n_out);
+}
+
+static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+                           const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                           const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t T,
+                           int32_t max_blocks, float* logits, float* layer_trace, int64_t stream) {
     const int W = m->cfg.width, dt = m->cfg.dtype;
     const float eps = m->cfg.norm_eps;
     const bool bf = m->bf16();
@@ -420,5 +445,56 @@ int mi355_hybrid_forward(void* mp, const uint32_t* tokens, const int64_t* positi
     }
     return 0;
 }
+
+int mi355_hybrid_forward(void* mp, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+                         const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                         const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t T,
+                         int32_t max_blocks, int32_t max_context_len, float* logits, float* layer_trace, int64_t stream) {
+    HModel* m = static_cast<HModel*>(mp);
+    HCHECK(forward_check(m, tokens, positions, slot_mapping, block_tables, context_lens, cu_seqlens_q, state_slots, out_rows, n_out,
+                         num_seqs, T, max_blocks, max_context_len, logits));
+    return forward_enqueue(m, tokens, positions, slot_mapping, block_tables, context_lens, cu_seqlens_q, state_slots, out_rows, n_out,
+                           num_seqs, T, max_blocks, logits, layer_trace, stream);
+}
+
+// The same step replayed from a hipGraph: the launches of a step depend on the counts and on the device pointers only (positions,
+// block tables and slots are read on the device), so a caller that keeps its step inputs in static device buffers -- as the llama
+// host layers' greedy loops do -- pays one graph launch per step instead of one launch per kernel.  `stream` must be a capturing-
+// capable (non-default) stream.  The first step of a shape runs eagerly inside the capture's instantiate-and-launch.
+int mi355_hybrid_forward_graph(void* mp, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+                               const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                               const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t T,
+                               int32_t max_blocks, int32_t max_context_len, float* logits, int64_t stream) {
+    HModel* m = static_cast<HModel*>(mp);
+    if (stream == 0) return -5;
+    HCHECK(forward_check(m, tokens, positions, slot_mapping, block_tables, context_lens, cu_seqlens_q, state_slots, out_rows, n_out,
+                         num_seqs, T, max_blocks, max_context_len, logits));
+    const std::vector<int64_t> key = {(int64_t)(intptr_t)tokens, (int64_t)(intptr_t)positions, (int64_t)(intptr_t)slot_mapping,
+                                      (int64_t)(intptr_t)block_tables, (int64_t)(intptr_t)context_lens, (int64_t)(intptr_t)cu_seqlens_q,
+                                      (int64_t)(intptr_t)state_slots, (int64_t)(intptr_t)out_rows, (int64_t)(intptr_t)logits,
+                                      n_out, num_seqs, T, max_blocks};
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    auto it = m->graphs.find(key);
+    if (it == m->graphs.end()) {
+        if (m->graphs.size() >= 256) drop_graphs(m);
+        HModel::StepGraph g;
+        HHIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+        const int rc = forward_enqueue(m, tokens, positions, slot_mapping, block_tables, context_lens, cu_seqlens_q, state_slots, out_rows,
+                                       n_out, num_seqs, T, max_blocks, logits, nullptr, stream);
+        const hipError_t e = hipStreamEndCapture(st, &g.graph);
+        if (rc != 0 || e != hipSuccess) { if (g.graph) (void)hipGraphDestroy(g.graph); return rc != 0 ? rc : (int)e; }
+        const hipError_t ei = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+        if (ei != hipSuccess) { (void)hipGraphDestroy(g.graph); return (int)ei; }
+        it = m->graphs.emplace(key, g).first;
+        ++m->graph_captures;
+    } else {
+        ++m->graph_replays;
+    }
+    HHIP(hipGraphLaunch(it->second.exec, st));
+    return 0;
+}
+
+int64_t mi355_hybrid_graph_captures(void* mp) { return mp ? static_cast<HModel*>(mp)->graph_captures : -1; }
+int64_t mi355_hybrid_graph_replays(void* mp) { return mp ? static_cast<HModel*>(mp)->graph_replays : -1; }
 
 }  // extern "C"

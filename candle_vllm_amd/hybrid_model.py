@@ -245,41 +245,94 @@ class HybridModel:
         return int(lib.mi355_hybrid_cache_bytes(self.h, int(num_blocks)))
 
     # ---- one step
-    def step(self, meta, state_slots, want_rows=None, trace=False, stream=None, sync=True):
+    GRAPH_MAX_TOKENS = 16                  # steps of up to this many tokens (decoding batches) replay a hipGraph; longer ones run eagerly
+
+    def _stage(self, total):
+        """pinned host + device staging of one step's inputs (one copy per step); grows, never shrinks"""
+        if getattr(self, "_dev", None) is None or self._dev.numel() < total:
+            n = max(2 * total, 1 << 16)
+            self._host = torch.empty(n, dtype=torch.uint8, pin_memory=True)
+            self._host_np = self._host.numpy()
+            self._dev = torch.empty(n, dtype=torch.uint8, device="cuda")
+            self._logits = {}
+        if getattr(self, "_stream", None) is None:
+            self._stream = torch.cuda.Stream()
+
+    def step(self, meta, state_slots, want_rows=None, trace=False, sync=True, graph=True):
         """meta: BlockEngine.prepare_prompt's dict (every sequence brings its not yet cached tokens: a prompt, a portion of one, or
         one decoded token); state_slots: the sequences' slots (BlockEngine.state_acquire); want_rows: token rows whose logits are
-        wanted (default: every sequence's last).  -> logits f32 [len(want_rows), vocab] (and the residual stream behind every layer
-        [n_layers, T, width] with trace=True)."""
-        dev = "cuda"
+        wanted (default: every sequence's last).  -> logits f32 [len(want_rows), vocab], valid until the next step of the same
+        shape (and the residual stream behind every layer [n_layers, T, width] with trace=True).  The step's inputs travel in one
+        copy into a static device buffer; steps of up to GRAPH_MAX_TOKENS tokens replay a captured hipGraph."""
         n = len(meta["context_lens"])
         T = len(meta["input_ids"])
         cu = np.asarray(meta["cu_seqlens_q"]).astype(np.int64)
         if want_rows is None:
             want_rows = (cu[1:] - 1).tolist()
         want = np.asarray(want_rows, np.int32)
+        n_out = len(want)
         max_ctx = int(meta["max_context_len"])
         self.ensure_rope(max_ctx)
-
-        def to(a, dt):
-            return torch.from_numpy(np.ascontiguousarray(np.asarray(a).astype(dt))).to(dev)
-        tok = to(np.asarray(meta["input_ids"]).astype(np.int64), np.int32)
-        pos, slots = to(meta["positions"], np.int64), to(meta["slot_mapping"], np.int64)
-        bt = to(np.asarray(meta["block_tables"]).astype(np.int64), np.int32).contiguous()
-        ctx, cuq = to(np.asarray(meta["context_lens"]).astype(np.int64), np.int32), to(cu, np.int32)
-        st = to(state_slots, np.int32)
-        if len(state_slots) != n or (len(state_slots) and (min(state_slots) < 0 or max(state_slots) >= self.state_slots)):
+        if len(state_slots) != n or (n and (min(state_slots) < 0 or max(state_slots) >= self.state_slots)):
             raise ValueError("every sequence of a step needs a state slot of the pool")
-        wr = to(want, np.int32) if len(want) else None
-        logits = torch.empty((len(want), self.vocab), dtype=torch.float32, device=dev)
-        tr = torch.empty((len(self.spec.layers), T, self.width), dtype=torch.float32, device=dev) if trace else None
-        s = torch.cuda.current_stream().cuda_stream if stream is None else stream
-        _check(lib.mi355_hybrid_forward(self.h, tok.data_ptr(), pos.data_ptr(), slots.data_ptr(), bt.data_ptr(), ctx.data_ptr(),
-                                        cuq.data_ptr(), st.data_ptr(), wr.data_ptr() if wr is not None else None, len(want), n, T,
-                                        bt.shape[1], max_ctx, logits.data_ptr() if len(want) else None,
-                                        tr.data_ptr() if trace else None, s), "hybrid_forward")
+        bt = np.asarray(meta["block_tables"]).astype(np.int64)
+        Wb = max(8, -(-bt.shape[1] // 8) * 8)                 # table width in steps of 8 blocks: few distinct shapes
+        Tc = max(16, 1 << max(0, T - 1).bit_length())
+        nc = max(n, self.state_slots)
+        sizes = [("tok", Tc * 4), ("pos", Tc * 8), ("slot", Tc * 8), ("want", Tc * 4), ("ctx", nc * 4), ("cu", (nc + 1) * 4),
+                 ("st", nc * 4), ("bt", nc * Wb * 4)]
+        off, total = {}, 0
+        for name, b in sizes:
+            off[name] = total
+            total += -(-b // 16) * 16
+        self._stage(total)
+        if getattr(self, "_pending", False):
+            self._stream.synchronize()
+        h = self._host_np
+
+        def put(name, a, dt):
+            a = np.ascontiguousarray(np.asarray(a).astype(dt)).reshape(-1)
+            h[off[name]:off[name] + a.nbytes] = a.view(np.uint8)
+        put("tok", np.asarray(meta["input_ids"]).astype(np.int64), np.int32)
+        put("pos", meta["positions"], np.int64)
+        put("slot", meta["slot_mapping"], np.int64)
+        put("want", want, np.int32)
+        put("ctx", np.asarray(meta["context_lens"]).astype(np.int64), np.int32)
+        put("cu", cu, np.int32)
+        put("st", state_slots, np.int32)
+        btw = np.zeros((n, Wb), np.int32)
+        btw[:, :bt.shape[1]] = bt
+        put("bt", btw, np.int32)
+        base = self._dev.data_ptr()
+        ptr = {k: base + v for k, v in off.items()}
+        use_graph = bool(graph) and not trace and T <= self.GRAPH_MAX_TOKENS
+        if use_graph:
+            logits = self._logits.get(n_out)
+            if logits is None:
+                logits = self._logits[n_out] = torch.empty((max(n_out, 1), self.vocab), dtype=torch.float32, device="cuda")
+        else:
+            logits = torch.empty((max(n_out, 1), self.vocab), dtype=torch.float32, device="cuda")
+        tr = torch.empty((len(self.spec.layers), T, self.width), dtype=torch.float32, device="cuda") if trace else None
+        with torch.cuda.stream(self._stream):
+            self._dev[:total].copy_(self._host[:total], non_blocking=True)
+            s = self._stream.cuda_stream
+            if use_graph:
+                _check(lib.mi355_hybrid_forward_graph(self.h, ptr["tok"], ptr["pos"], ptr["slot"], ptr["bt"], ptr["ctx"], ptr["cu"], ptr["st"],
+                                                      ptr["want"], n_out, n, T, Wb, max_ctx, logits.data_ptr(), s), "hybrid_forward_graph")
+            else:
+                _check(lib.mi355_hybrid_forward(self.h, ptr["tok"], ptr["pos"], ptr["slot"], ptr["bt"], ptr["ctx"], ptr["cu"], ptr["st"],
+                                                ptr["want"], n_out, n, T, Wb, max_ctx, logits.data_ptr(),
+                                                tr.data_ptr() if trace else None, s), "hybrid_forward")
+        self._pending = True
         if sync:
-            torch.cuda.synchronize()
+            self._stream.synchronize()
+            self._pending = False
+        logits = logits[:n_out]
         return (logits, tr) if trace else logits
+
+    def graph_stats(self):
+        """(step graphs captured, steps replayed from one)"""
+        return int(lib.mi355_hybrid_graph_captures(self.h)), int(lib.mi355_hybrid_graph_replays(self.h))
 
     def forward_prefill(self, meta, state_slots):
         """logits of the last new token of every sequence (the prompt step of the engine loop)"""

@@ -19,6 +19,7 @@ class StepEngine:
         self.be.state_init(model.state_slots)
         model.alloc_cache(self.num_blocks)
         self.seqs, self._next = {}, 0
+        self.use_graph = True                 # short steps (decoding batches) replay a captured hipGraph
 
     def feed(self, rid, tokens):
         """admit `rid` with its first tokens, or append tokens to it; pages are taken for exactly what the sequence holds"""
@@ -64,7 +65,7 @@ class StepEngine:
                         raise ValueError("a wanted place outside the entry's tokens")
                     rows.append(int(cu[i] + k))
         slots = [self.be.state_slot(s) for s in group]
-        out = self.model.step(meta, slots, want_rows=rows, trace=trace)
+        out = self.model.step(meta, slots, want_rows=rows, trace=trace, graph=self.use_graph)
         for s in group:
             s.set_num_cached_tokens(s.get_len())
         return out

@@ -108,6 +108,15 @@ int mi355_hybrid_forward(void* model, const uint32_t* tokens, const int64_t* pos
                          const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs, int32_t num_tokens,
                          int32_t max_blocks, int32_t max_context_len, float* logits, float* layer_trace, int64_t stream);
 
+/* the same step from a hipGraph keyed by the device pointers and the counts (the caller keeps its step inputs in static device
+ * buffers); `stream` must not be the default stream; no layer trace */
+int mi355_hybrid_forward_graph(void* model, const uint32_t* tokens, const int64_t* positions, const int64_t* slot_mapping,
+                               const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                               const int32_t* state_slots, const int32_t* out_rows, int32_t n_out, int32_t num_seqs,
+                               int32_t num_tokens, int32_t max_blocks, int32_t max_context_len, float* logits, int64_t stream);
+int64_t mi355_hybrid_graph_captures(void* model);
+int64_t mi355_hybrid_graph_replays(void* model);
+
 /* ---- the mechanisms alone (tests, other host layers).  `dtype` is the type of 16/32-bit operands marked (dt); the rest is f32 */
 /* token_seq i32 [T]: the sequence (row of cu_seqlens_q) of every token row */
 int mi355_hyb_token_seq(int32_t* token_seq, const uint32_t* cu_seqlens_q, int32_t num_seqs, int64_t stream);

@@ -83,6 +83,16 @@ def test_registry_picks_the_host_layer_by_config(tmp_path, lib):
         registry.load_model(str(tmp_path))
 
 
+def test_llama_checkpoint_names_map_to_dense_slots(lib):
+    from candle_vllm_amd import dense_loader as dl
+    assert dl.slot_of("model.layers.11.self_attn.k_proj.weight") == (11, "wk")
+    assert dl.slot_of("model.layers.0.mlp.up_proj.weight") == (0, "w3") and dl.slot_of("lm_head.weight") == (-1, "output")
+    assert dl.slot_of("model.layers.3.self_attn.rotary_emb.inv_freq") is None
+    d = dl.dims_from_config({"hidden_size": 64, "num_hidden_layers": 2, "num_attention_heads": 4, "num_key_value_heads": 2,
+                             "intermediate_size": 128, "vocab_size": 99, "rms_norm_eps": 1e-6, "architectures": ["Qwen2ForCausalLM"]})
+    assert (d.head_dim, d.n_kv_heads, d.qkv_bias, d.rms_eps) == (16, 2, True, 1e-6)
+
+
 def test_state_slots_follow_the_sequences(lib):
     from candle_vllm_amd.block_engine import BlockEngine
     be = BlockEngine(4, 8, 0)

@@ -463,6 +463,34 @@ def test_long_decoding_and_first_tokens(lib):
     assert row_err(np.concatenate(rows), want) < TOL["float32"]
 
 
+def test_graph_replays_equal_eager_steps(lib):
+    """decoding batches replay a captured hipGraph: every replay, with eager prompt portions of other requests between them, gives the
+    eager step's logits bit for bit"""
+    _gpu()
+    from candle_vllm_amd.step_engine import StepEngine
+    cfg = small_config(0)
+    m, W = build(cfg, "bfloat16", seed=12)
+    rng = np.random.default_rng(13)
+    toks = {r: rng.integers(0, cfg["vocab"], 60).tolist() for r in "ab"}
+    outs = {}
+    for use_graph in (False, True):
+        eng = StepEngine(m, 256)
+        eng.use_graph = use_graph
+        rows = []
+        eng.feed("a", toks["a"][:20]); eng.feed("b", toks["b"][:33])
+        rows.append(eng.step(["a", "b"]).cpu().numpy())
+        for i in range(20):
+            eng.feed("a", toks["a"][20 + i:21 + i]); eng.feed("b", toks["b"][33 + i:34 + i])
+            rows.append(eng.step(["a", "b"]).cpu().numpy())
+            if i == 7:                                                      # an eager prompt of a third request between two replays
+                eng.feed("c", toks["a"][:25]); rows.append(eng.step(["c"]).cpu().numpy()); eng.finish("c")
+        eng.finish("a"); eng.finish("b")
+        outs[use_graph] = np.concatenate(rows)
+    assert np.array_equal(outs[False], outs[True])
+    cap, rep = m.graph_stats()
+    assert cap >= 1 and rep >= 15
+
+
 @pytest.mark.parametrize("chunk", [0, 7])
 def test_greedy_generation_through_scheduler(lib, chunk):
     """run_engine + the C++ scheduler (continuous batching, staggered arrivals, chunked prefill): every request generates exactly the
