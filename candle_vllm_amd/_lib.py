@@ -385,7 +385,7 @@ _sig("mi355_hyb_delta_rule", ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp
                                               c_vp] + [c_i32] * 6 + [c_f32, c_vp, c_i64])
 _sig("mi355_hyb_delta_rule_scratch_floats", ctypes.c_int, [c_i32] * 5)
 _sig("mi355_hyb_gated_norm", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_i64])
-_sig("mi355_hyb_mingru", ctypes.c_int, [c_vp, c_i32, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_mingru", ctypes.c_int, [c_vp, c_i32, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_clamped_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_f32, c_f32, c_i64])
 
 # the hand-written ctypes mirrors must have the layout the library was built with

@@ -378,7 +378,7 @@ struct AttnArgs {
     void* out; int ldo, out_off;
     const void* q; const void* k_pages; const void* v_pages;
     const uint32_t* bt; const uint32_t* ctx; const uint32_t* cu_q; const int32_t* tok_seq; const float* sink;
-    int n_seqs, H, G, d, vd, bs, max_blocks, window; float scale, out_scale; int cp2;
+    int n_seqs, H, G, d, vd, bs, max_blocks, window; float scale, out_scale; int cp2, out_f32;
 };
 // 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
 template <typename TC> struct Vec16;
@@ -403,7 +403,8 @@ template <> struct Vec16<float> {
 // partial results are merged through LDS.  The sink enters the merge as a partial result with maximum sink, denominator 1 and no
 // value.  VEC (head sizes that are multiples of 16 bytes): rows are read 16 bytes at a time; for the value sum the wave's lanes
 // are (key, 16-byte chunk of the row) pairs -- 64 / cp2 keys per pass -- and the keys' partial sums are added by lane exchanges.
-template <typename TC, typename TO, int NW, bool VEC> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
+// DQ > 0 (VEC, d = DQ): the query sits in registers, so a key's score costs its 16-byte loads and d FMAs and nothing else.
+template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
     constexpr int EPV = Vec16<TC>::N;
     constexpr int NACC = VEC ? EPV : 8;
     extern __shared__ __align__(16) float smem[];
@@ -420,6 +421,11 @@ template <typename TC, typename TO, int NW, bool VEC> __global__ __launch_bounds
     const TC* q = static_cast<const TC*>(p.q) + ((size_t)t * p.H + h) * p.d;
     for (int i = threadIdx.x; i < p.d; i += blockDim.x) qs[i] = ld<TC>(q, i);
     __syncthreads();
+    float qr[DQ > 0 ? DQ : 1];
+    if (DQ > 0) {
+#pragma unroll
+        for (int i = 0; i < DQ; ++i) qr[i] = qs[i];
+    }
     const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
     const int cp2 = p.cp2, chunk = lane & (cp2 - 1), ksub = lane / cp2, kpp = 64 / cp2;     // VEC only
     const bool chunk_ok = chunk * EPV < p.vd;
@@ -434,7 +440,15 @@ template <typename TC, typename TO, int NW, bool VEC> __global__ __launch_bounds
             page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
             const TC* kr = static_cast<const TC*>(p.k_pages) + ((size_t)page_row * p.G + g) * p.d;
             float dot = 0.f;
-            if (VEC) {
+            if (VEC && DQ > 0) {
+#pragma unroll
+                for (int i = 0; i < DQ; i += EPV) {
+                    float x[EPV];
+                    Vec16<TC>::load(kr + i, x);
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) dot = fmaf(qr[i + e], x[e], dot);
+                }
+            } else if (VEC) {
                 for (int i = 0; i < p.d; i += EPV) {
                     float x[EPV];
                     Vec16<TC>::load(kr + i, x);
@@ -495,11 +509,12 @@ template <typename TC, typename TO, int NW, bool VEC> __global__ __launch_bounds
         float L = p.sink ? expf(p.sink[h] - M) : 0.f;
         float cw[NW];
         for (int w = 0; w < NW; ++w) { cw[w] = pm[w] == -INFINITY ? 0.f : expf(pm[w] - M); L += pl[w] * cw[w]; }
-        TO* out = static_cast<TO*>(p.out) + (size_t)t * p.ldo + p.out_off + (size_t)h * p.vd;
+        const size_t base = (size_t)t * p.ldo + p.out_off + (size_t)h * p.vd;
         for (int col = lane; col < p.vd; col += 64) {
             float o = 0.f;
             for (int w = 0; w < NW; ++w) o += pacc[w * p.vd + col] * cw[w];
-            st<TO>(out, col, o / L * p.out_scale);
+            if (p.out_f32) st<float>(static_cast<float*>(p.out), base + col, o / L * p.out_scale);
+            else st<uint16_t>(static_cast<uint16_t*>(p.out), base + col, o / L * p.out_scale);
         }
     }
 }
@@ -735,6 +750,55 @@ template <typename TO, int UNR> __global__ __launch_bounds__(64) void mingru_ker
     stt[c] = S;
 }
 
+// Long portions: S_t = (1 - z_t) S_(t-1) + z_t c_t is a composition of affine maps, so the portion is cut into NSEG segments, one wave
+// each: pass 1 reduces a segment to (A, B) with S_end = A S_start + B, the waves exchange (A, B) through LDS, every wave folds the
+// segments before its own into its starting state and walks its segment again writing the outputs.
+template <typename TO, int NSEG, int UNR> __global__ __launch_bounds__(64 * NSEG) void mingru_seg_kernel(GruArgs p) {
+    __shared__ float sA[NSEG][64], sB[NSEG][64];
+    const int s = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.x * 64 + lane;
+    const int tb = (int)p.cu_q[s], te = (int)p.cu_q[s + 1];
+    if (te <= tb) return;
+    const bool ok_ = c < p.width;
+    const int cc = ok_ ? c : 0;
+    const int seg = (te - tb + NSEG - 1) / NSEG;
+    const int lo = min(te, tb + w * seg), hi = min(te, lo + seg);
+    float A = 1.f, B = 0.f;
+    for (int t0 = lo; t0 < hi; t0 += UNR) {
+        float z[UNR], u[UNR];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) { const float* row = p.proj + (size_t)min(t0 + k, hi - 1) * p.ldp; z[k] = row[p.z_off + cc]; u[k] = row[p.x_off + cc]; }
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            if (t0 + k >= hi) break;
+            const float zz = sigmoidf_(z[k]), cand = u[k] >= 0.f ? u[k] + 0.5f : sigmoidf_(u[k]);
+            A *= (1.f - zz);
+            B = (1.f - zz) * B + zz * cand;
+        }
+    }
+    sA[w][lane] = A; sB[w][lane] = B;
+    __syncthreads();
+    const int start_pos = (int)p.ctx[s] - (te - tb);
+    float* stt = p.state + (size_t)p.slots[s] * p.state_stride;
+    float S = (start_pos > 0 && ok_) ? stt[cc] : 0.f;
+    for (int v = 0; v < w; ++v) S = sA[v][lane] * S + sB[v][lane];
+    for (int t0 = lo; t0 < hi; t0 += UNR) {
+        float z[UNR], u[UNR], gg[UNR];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            const float* row = p.proj + (size_t)min(t0 + k, hi - 1) * p.ldp;
+            z[k] = row[p.z_off + cc]; u[k] = row[p.x_off + cc]; gg[k] = row[p.g_off + cc];
+        }
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            if (t0 + k >= hi) break;
+            const float zz = sigmoidf_(z[k]), cand = u[k] >= 0.f ? u[k] + 0.5f : sigmoidf_(u[k]);
+            S = (1.f - zz) * S + zz * cand;
+            if (ok_) st<TO>(static_cast<TO*>(p.out), (size_t)(t0 + k) * p.width + c, S * siluf_(gg[k]));
+        }
+    }
+    if (w == NSEG - 1 && ok_) stt[c] = S;
+}
+
 __global__ void token_seq_kernel(int32_t* tok_seq, const uint32_t* cu_q, int n_seqs) {
     const int s = blockIdx.x;
     for (int t = (int)cu_q[s] + threadIdx.x; t < (int)cu_q[s + 1]; t += blockDim.x) tok_seq[t] = s;
@@ -873,21 +937,26 @@ int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
     if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return -1;
     if (block_size <= 0 || max_blocks <= 0 || window < 0) return -1;
     if (T <= 0) return 0;
+    const bool f = dtype == MI355_DTYPE_F32;
     AttnArgs p{out, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq, sink,
-               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale, 64};
-    constexpr int NW = 4;
-    const size_t lds = (size_t)(((dim + 3) & ~3) + 2 * NW + NW * vdim) * sizeof(float);
+               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale, 64, out_dtype == MI355_DTYPE_F32};
     const dim3 grid(T, heads);
     hipStream_t s_ = to_stream(stream);
-    const bool f = dtype == MI355_DTYPE_F32, of = out_dtype == MI355_DTYPE_F32;
     const int epv = f ? 4 : 8;
     const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0;
     if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; }
     else if (vdim > 512) return -1;
-#define WA(TC, TO) do { if (vec) window_attention_kernel<TC, TO, NW, true><<<grid, 64 * NW, lds, s_>>>(p); \
-                        else window_attention_kernel<TC, TO, NW, false><<<grid, 64 * NW, lds, s_>>>(p); } while (0)
-    if (f && of) WA(float, float); else if (f) WA(float, uint16_t); else if (of) WA(uint16_t, float); else WA(uint16_t, uint16_t);
+    // few (token, head) pairs (decoding batches): eight waves share a window instead of four
+    const bool wide = (int64_t)T * heads < 2048;
+    const int dq = !vec ? 0 : dim == 64 ? 64 : dim == 128 ? 128 : 0;
+#define WA3(TC, NW, VEC, DQ) window_attention_kernel<TC, NW, VEC, DQ><<<grid, 64 * NW, (size_t)(((dim + 3) & ~3) + 2 * NW + NW * vdim) * sizeof(float), s_>>>(p)
+#define WA2(TC, NW) do { if (!vec) WA3(TC, NW, false, 0); else if (dq == 64) WA3(TC, NW, true, 64); else if (dq == 128) WA3(TC, NW, true, 128); \
+                         else WA3(TC, NW, true, 0); } while (0)
+#define WA(TC) do { if (wide) WA2(TC, 8); else WA2(TC, 4); } while (0)
+    if (f) WA(float); else WA(uint16_t);
 #undef WA
+#undef WA2
+#undef WA3
     LAUNCH_OK(); return 0;
 }
 
@@ -956,11 +1025,16 @@ int mi355_hyb_gated_norm(void* out, int32_t out_dtype, int32_t ldo, int32_t out_
 
 int mi355_hyb_mingru(void* out, int32_t out_dtype, float* state, int64_t state_stride, const float* proj, int32_t ldp, int32_t z_off,
                      int32_t x_off, int32_t g_off, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
-                     const int32_t* state_slots, int32_t num_seqs, int32_t width, int64_t stream) {
+                     const int32_t* state_slots, int32_t num_seqs, int32_t num_tokens, int32_t width, int64_t stream) {
     if (!out || !state || !proj || !context_lens || !cu_seqlens_q || !state_slots || !is_dt(out_dtype) || width <= 0) return -1;
     if (num_seqs <= 0) return 0;
     GruArgs p{out, state, state_stride, proj, ldp, z_off, x_off, g_off, context_lens, cu_seqlens_q, state_slots, width};
     const dim3 grid((width + 63) / 64, num_seqs);
+    if (num_tokens >= 256) {                            // some portion may be long: segmented scan
+        if (out_dtype == MI355_DTYPE_F32) mingru_seg_kernel<float, 16, 4><<<grid, 1024, 0, to_stream(stream)>>>(p);
+        else mingru_seg_kernel<uint16_t, 16, 4><<<grid, 1024, 0, to_stream(stream)>>>(p);
+        LAUNCH_OK(); return 0;
+    }
     if (out_dtype == MI355_DTYPE_F32) mingru_kernel<float, 8><<<grid, 64, 0, to_stream(stream)>>>(p);
     else mingru_kernel<uint16_t, 8><<<grid, 64, 0, to_stream(stream)>>>(p);
     LAUNCH_OK(); return 0;

@@ -427,7 +427,7 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
         }
         if (c.mixer == MI355_HYB_MIX_MINGRU)
             HCHECK(mi355_hyb_mingru(m->mix, dt, m->state + L.state_off, m->slot_floats, m->proj, ldp, L.off[0], L.off[1], L.off[2],
-                                    context_lens, cu_seqlens_q, state_slots, num_seqs, c.g_width, stream));
+                                    context_lens, cu_seqlens_q, state_slots, num_seqs, T, c.g_width, stream));
         HCHECK(mi355_hyb_linear(m->y, W, m->mix, dt, L.out_k, L.w[MI355_HW_OUT_PROJ].p, nullptr, T, W, L.out_k, dt, stream));
         HCHECK(mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(MI355_HW_NORM1), T, W, eps, stream));
         if (c.mlp_kind) {

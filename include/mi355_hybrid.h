@@ -177,7 +177,7 @@ int mi355_hyb_gated_norm(void* out, int32_t out_dtype, int32_t ldo, int32_t out_
  * S = (1 - z) S + z candidate, out (dt_out) [T, width] = S silu(proj[:, g_off + c]); state f32 [slots] x [width] */
 int mi355_hyb_mingru(void* out, int32_t out_dtype, float* state, int64_t state_stride, const float* proj, int32_t ldp, int32_t z_off,
                      int32_t x_off, int32_t g_off, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
-                     const int32_t* state_slots, int32_t num_seqs, int32_t width, int64_t stream);
+                     const int32_t* state_slots, int32_t num_seqs, int32_t num_tokens, int32_t width, int64_t stream);
 /* out (dt_out) [T, ff] = g sigmoid(alpha g) (u + 1), g = min(gu[:, j], limit), u = clamp(gu[:, ff + j], -limit, limit) */
 int mi355_hyb_clamped_glu(void* out, int32_t out_dtype, const float* gu, int32_t num_tokens, int32_t ff, float limit, float alpha,
                           int64_t stream);

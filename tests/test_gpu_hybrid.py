@@ -286,19 +286,19 @@ def test_gated_norm_and_mingru(lib):
         want = H.rms_norm(f(o), f(w), 1e-5) * act(f(gi)[:, :Hh * vd].reshape(T, Hh, vd)) * 0.25
         assert np.abs(out.cpu().numpy()[:, 3:].reshape(T, Hh, vd) - want).max() < 5e-6
     width, ldp = 70, 3 * 70 + 1
-    proj = f(2 * rng.standard_normal((40, ldp)))
-    want, S_want = H.min_gru(proj[:, 1:1 + width], proj[:, 1 + width:1 + 2 * width])
-    want = want * H.silu(proj[:, 1 + 2 * width:1 + 3 * width])
-    state = dev(rng.standard_normal((3, width + 4)))
-    got = []
-    for lo, hi in ((0, 2), (2, 3), (3, 20), (20, 40)):
-        out = torch.zeros((hi - lo, width), device="cuda")
-        ok(lib.mi355_hyb_mingru(out.data_ptr(), F32, state.data_ptr(), width + 4, P(proj[lo:hi]), ldp, 1, 1 + width, 1 + 2 * width,
-                                P([hi], np.int32), P([0, hi - lo], np.int32), P([2], np.int32), 1, width,
-                                _st()))
-        got.append(out.cpu().numpy())
-    assert np.abs(np.concatenate(got) - want).max() < 1e-5
-    assert np.abs(state.cpu().numpy()[2, :width] - S_want).max() < 1e-5
+    for n_tok, cuts in ((40, ((0, 2), (2, 3), (3, 20), (20, 40))), (700, ((0, 300), (300, 301), (301, 700)))):   # short portions: plain scan;
+        proj = f(2 * rng.standard_normal((n_tok, ldp)))                                                      # long ones: segmented scan
+        want, S_want = H.min_gru(proj[:, 1:1 + width], proj[:, 1 + width:1 + 2 * width])
+        want = want * H.silu(proj[:, 1 + 2 * width:1 + 3 * width])
+        state = dev(rng.standard_normal((3, width + 4)))
+        got = []
+        for lo, hi in cuts:
+            out = torch.zeros((hi - lo, width), device="cuda")
+            ok(lib.mi355_hyb_mingru(out.data_ptr(), F32, state.data_ptr(), width + 4, P(proj[lo:hi]), ldp, 1, 1 + width, 1 + 2 * width,
+                                    P([hi], np.int32), P([0, hi - lo], np.int32), P([2], np.int32), 1, hi - lo, width, _st()))
+            got.append(out.cpu().numpy())
+        assert np.abs(np.concatenate(got) - want).max() < 2e-5
+        assert np.abs(state.cpu().numpy()[2, :width] - S_want).max() < 2e-5
 
 
 # ------------------------------------------------------------------------------------------------------------ whole models
