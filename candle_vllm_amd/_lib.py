@@ -379,6 +379,7 @@ _sig("mi355_hyb_linear", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c
 _sig("mi355_hyb_norm_add", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_f32, c_i64])
 _sig("mi355_hyb_attn_prepare", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_vp] * 6 + [c_i32] * 6 + [c_f32, c_i32, c_i64])
 _sig("mi355_hyb_window_attention", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 8 + [c_i32] * 9 + [c_f32, c_f32, c_i32, c_i64])
+_sig("mi355_hyb_set_attention_mfma", None, [c_i32])
 _sig("mi355_hyb_conv_silu", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 4 + [c_i64])
 _sig("mi355_hyb_conv_state_update", ctypes.c_int, [c_vp, c_i64, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_delta_rule", ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_vp,

@@ -519,6 +519,145 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
     }
 }
 
+// Prompt-sized steps, bf16 pages: one wave per (tile of 16 consecutive new tokens of one sequence, head), 64 keys per iteration.
+//   S = Q K^T on the matrix cores: the query tile's fragments stay in registers, a key's fragments come straight from its page row
+//   (lane (m16, kg) = 16 bytes of key m16 of a 16-key tile); the accumulator holds queries 4 kg + v against key m16.
+//   Mask, scale and the online softmax run on that layout in f32 (row maxima / sums: exchanges among the 16 lanes of a kg group).
+//   P V: the probabilities go through LDS into A-fragment order as TWO bf16 planes (p = hi + lo, so the weights keep about 16 bits
+//   of mantissa), the 64 value rows are transposed through LDS ([column][key]) so that a B fragment is one 16-byte read.
+// The sink is applied at the end: denominator += exp(sink - max).
+template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention_mfma_kernel(AttnArgs p) {
+    constexpr int RS = 72;                                           // bf16 per LDS row: 64 keys + 8 of padding (144 bytes)
+    __shared__ __align__(16) uint16_t Ph[16 * RS], Pl[16 * RS], Vt[VT * 16 * RS];
+    const int lane = threadIdx.x, m16 = lane & 15, kg = lane >> 4;
+    int b = blockIdx.x, s = 0, n_new = 0;
+    for (; s < p.n_seqs; ++s) {
+        n_new = (int)(p.cu_q[s + 1] - p.cu_q[s]);
+        const int tiles = (n_new + 15) >> 4;
+        if (b < tiles) break;
+        b -= tiles;
+    }
+    if (s >= p.n_seqs) return;
+    const int t0 = (int)p.cu_q[s] + b * 16, nq = min(16, (int)p.cu_q[s + 1] - t0);
+    const int pos0 = (int)p.ctx[s] - n_new + b * 16;
+    const int h = blockIdx.y, g = h / (p.H / p.G), d = p.d, vd = p.vd;
+    const uint16_t* Q = static_cast<const uint16_t*>(p.q);
+    const uint16_t* K = static_cast<const uint16_t*>(p.k_pages);
+    const uint16_t* V = static_cast<const uint16_t*>(p.v_pages);
+    const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
+    uint4 qf[DK];
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks)
+        qf[ks] = m16 < nq ? *reinterpret_cast<const uint4*>(Q + ((size_t)(t0 + m16) * p.H + h) * d + ks * 32 + 8 * kg) : uint4{0, 0, 0, 0};
+    float mrow[4], lrow[4];
+    f32x4_t acc[VT];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { mrow[v] = -INFINITY; lrow[v] = 0.f; }
+#pragma unroll
+    for (int c = 0; c < VT; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int hi = pos0 + nq - 1;
+    const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+    for (int j0 = lo; j0 <= hi; j0 += 64) {
+        f32x4_t sacc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            sacc[kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            const int key = j0 + kt * 16 + m16;
+            const bool kv = key <= hi;
+            const size_t pr = kv ? (size_t)bt[key / p.bs] * p.bs + (key % p.bs) : 0;
+            const uint16_t* kr = K + (pr * p.G + g) * d + 8 * kg;
+#pragma unroll
+            for (int ks = 0; ks < DK; ++ks) {
+                const uint4 kf = kv ? *reinterpret_cast<const uint4*>(kr + ks * 32) : uint4{0, 0, 0, 0};
+                sacc[kt] = mfma_bf16(qf[ks], kf, sacc[kt]);
+            }
+        }
+        // the 64 value rows of this chunk, transposed into LDS (zeros past the end: a stale NaN times a zero weight would poison the sum)
+        {
+            const int key = j0 + lane;
+            const bool kv = key <= hi;
+            const size_t pr = kv ? (size_t)bt[key / p.bs] * p.bs + (key % p.bs) : 0;
+            const uint16_t* vr = V + (pr * p.G + g) * vd;
+#pragma unroll
+            for (int c8 = 0; c8 < VT * 2; ++c8) {
+                const uint4 x = kv ? *reinterpret_cast<const uint4*>(vr + c8 * 8) : uint4{0, 0, 0, 0};
+                const uint32_t w[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    Vt[(c8 * 8 + 2 * e) * RS + lane] = (uint16_t)(w[e] & 0xFFFFu);
+                    Vt[(c8 * 8 + 2 * e + 1) * RS + lane] = (uint16_t)(w[e] >> 16);
+                }
+            }
+        }
+        // mask, scale, online softmax (rows 4 kg + v; this lane's keys: kt * 16 + m16)
+        float mx[4], sc[4][4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = 4 * kg + v, qpos = pos0 + r;
+            mx[v] = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                const int key = j0 + kt * 16 + m16;
+                const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window);
+                sc[v][kt] = ok_ ? sacc[kt][v] * p.scale : -INFINITY;
+                mx[v] = fmaxf(mx[v], sc[v][kt]);
+            }
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) mx[v] = fmaxf(mx[v], __shfl_xor(mx[v], o));
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float mn = fmaxf(mrow[v], mx[v]);
+            const float corr = (mn == -INFINITY || mrow[v] == -INFINITY) ? (mn == -INFINITY ? 1.f : 0.f) : expf(mrow[v] - mn);
+            float rs = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                const float pv = sc[v][kt] == -INFINITY ? 0.f : expf(sc[v][kt] - mn);
+                rs += pv;
+                const uint16_t ph = f32_to_bf16(pv);
+                Ph[(4 * kg + v) * RS + kt * 16 + m16] = ph;
+                Pl[(4 * kg + v) * RS + kt * 16 + m16] = f32_to_bf16(pv - bf16_to_f32(ph));
+            }
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) rs += __shfl_xor(rs, o);
+            lrow[v] = lrow[v] * corr + rs;
+            mrow[v] = mn;
+#pragma unroll
+            for (int c = 0; c < VT; ++c) acc[c][v] *= corr;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2) {
+            const uint4 ah = *reinterpret_cast<const uint4*>(&Ph[m16 * RS + k2 * 32 + 8 * kg]);
+            const uint4 al = *reinterpret_cast<const uint4*>(&Pl[m16 * RS + k2 * 32 + 8 * kg]);
+#pragma unroll
+            for (int c = 0; c < VT; ++c) {
+                const uint4 vf = *reinterpret_cast<const uint4*>(&Vt[(c * 16 + m16) * RS + k2 * 32 + 8 * kg]);
+                acc[c] = mfma_bf16(ah, vf, acc[c]);
+                acc[c] = mfma_bf16(al, vf, acc[c]);
+            }
+        }
+        __syncthreads();
+    }
+    const float sink = p.sink ? p.sink[h] : -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int r = 4 * kg + v;
+        if (r >= nq) continue;
+        const float M = fmaxf(mrow[v], sink);
+        const float cm = expf(mrow[v] - M);
+        const float L = lrow[v] * cm + (p.sink ? expf(sink - M) : 0.f);
+        const float f = cm / L * p.out_scale;
+        const size_t base = (size_t)(t0 + r) * p.ldo + p.out_off + (size_t)h * vd;
+#pragma unroll
+        for (int c = 0; c < VT; ++c) {
+            const float o = acc[c][v] * f;
+            if (p.out_f32) static_cast<float*>(p.out)[base + c * 16 + m16] = o;
+            else static_cast<uint16_t*>(p.out)[base + c * 16 + m16] = f32_to_bf16(o);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------------------ short convolution
 struct ConvArgs {
     float* out; const float* proj; int ldp, off; const float* w; float* state; int64_t state_stride;
@@ -816,6 +955,8 @@ __global__ void fill_f32_kernel(float* out, float v, int64_t n) {
     if (i < n) out[i] = v;
 }
 
+int g_attn_mfma = 1;            // mi355_hyb_set_attention_mfma(0): prompt steps take the generic kernel too (A/B, tests of both paths)
+
 #define LAUNCH_OK() do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)
 inline bool is_dt(int dt) { return dt == MI355_DTYPE_F32 || dt == MI355_DTYPE_BF16; }
 
@@ -829,6 +970,7 @@ int mi355_hyb_token_seq(int32_t* tok_seq, const uint32_t* cu_seqlens_q, int32_t 
     token_seq_kernel<<<num_seqs, 64, 0, to_stream(stream)>>>(tok_seq, cu_seqlens_q, num_seqs);
     LAUNCH_OK(); return 0;
 }
+void mi355_hyb_set_attention_mfma(int32_t on) { g_attn_mfma = on ? 1 : 0; }
 int mi355_hyb_bf16_to_f32(float* out, const uint16_t* in, int64_t n, int64_t stream) {
     if (n <= 0) return 0;
     bf16_to_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(out, in, n);
@@ -946,6 +1088,22 @@ int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
     const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0;
     if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; }
     else if (vdim > 512) return -1;
+    // prompt-sized steps over bf16 pages: the matrix-core kernel (a tile of 16 tokens never spans two sequences)
+    if (!f && T >= 64 && dim % 32 == 0 && dim <= 256 && vdim % 16 == 0 && vdim <= 256 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
+        (uintptr_t)v_pages % 16 == 0 && g_attn_mfma) {
+        const dim3 mgrid((T + 15) / 16 + num_seqs, heads);
+        const int dk = dim / 32, vt = vdim / 16;
+#define WM(DK, VT) window_attention_mfma_kernel<DK, VT><<<mgrid, 64, 0, s_>>>(p)
+#define WMV(DK) do { if (vt <= 2) { if (vt == 1) WM(DK, 1); else WM(DK, 2); } else if (vt <= 4) { if (vt == 3) WM(DK, 3); else WM(DK, 4); } \
+                     else if (vt <= 8) { if (vt <= 6) { if (vt == 5) WM(DK, 5); else WM(DK, 6); } else { if (vt == 7) WM(DK, 7); else WM(DK, 8); } } \
+                     else ok_shape = false; } while (0)
+        bool ok_shape = true;
+        switch (dk) { case 1: WMV(1); break; case 2: WMV(2); break; case 3: WMV(3); break; case 4: WMV(4); break; case 6: WMV(6); break;
+                      case 8: WMV(8); break; default: ok_shape = false; }
+#undef WMV
+#undef WM
+        if (ok_shape) { LAUNCH_OK(); return 0; }
+    }
     // few (token, head) pairs (decoding batches): eight waves share a window instead of four
     const bool wide = (int64_t)T * heads < 2048;
     const int dq = !vec ? 0 : dim == 64 ? 64 : dim == 128 ? 128 : 0;

@@ -148,6 +148,8 @@ int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
                                const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, int32_t num_seqs, int32_t num_tokens,
                                int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size, int32_t max_blocks,
                                int32_t window, float scale, float out_scale, int32_t dtype, int64_t stream);
+/* 0: prompt-sized steps over bf16 pages take the generic kernel instead of the matrix-core one (A/B switch, process-wide; default 1) */
+void mi355_hyb_set_attention_mfma(int32_t on);
 /* short causal convolution over time per channel, then silu: out f32 [T, channels] from proj columns [off, off + channels);
  * the taps - 1 inputs before a portion come from conv_state f32 [slots, channels, taps - 1] (zeros at position 0);
  * mi355_hyb_conv_state_update then moves the state behind the portion */
