@@ -745,17 +745,36 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(DeltaArgs p, float* prep
     if (lane == 0) out[b_off + h] = sigmoidf_(p.proj[(size_t)t * p.ldp + p.b_off + h]);
 }
 
-// The scan.  A workgroup of 256 threads owns 64 columns of one (sequence, head)'s state S [d, vd]; four neighbouring lanes share a
-// column, each holding DP = ceil(d / 4) of its rows in registers, and walk the new tokens in order:
+// sum over the LPC neighbouring lanes that share a state column
+// (data-parallel-primitive moves inside a row of 16 lanes: swap inside pairs, swap pairs inside quads, mirror inside half rows,
+// mirror inside the row -- after each add every lane holds the sum of twice as many lanes; no LDS traffic, a few cycles each)
+template <int CTRL> __device__ __forceinline__ float dpp_move(float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
+}
+template <int LPC> __device__ __forceinline__ float column_sum(float x) {
+    static_assert(LPC == 4 || LPC == 16, "a column is shared by a quad or by a row of 16 lanes");
+    x += dpp_move<0xB1>(x);                      // quad_perm [1, 0, 3, 2]
+    x += dpp_move<0x4E>(x);                      // quad_perm [2, 3, 0, 1]
+    if (LPC == 16) {
+        x += dpp_move<0x141>(x);                 // row_half_mirror
+        x += dpp_move<0x140>(x);                 // row_mirror
+    }
+    return x;
+}
+
+// The scan.  A workgroup of 256 threads owns 256 / LPC columns of one (sequence, head)'s state S [d, vd]; LPC neighbouring lanes share
+// a column, each holding DP = ceil(d / LPC) of its rows in registers, and walk the new tokens in order:
 //   S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
-// (the two sums over d are finished by two lane exchanges inside the quad).  q, k, g of CH tokens at a time sit in LDS, rows padded
-// so that the four parts fall into different banks; the next CH tokens are fetched into registers while the current ones are used.
-template <int DP, int CH> __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs p, const float* __restrict__ prep, int P) {
-    constexpr int RS = DP + 4, TOT = CH * 4 * DP, NPT = (TOT + 255) / 256;
-    __shared__ __align__(16) float sq[2][CH][4][RS], sk[2][CH][4][RS], sg[2][CH][4][RS];
+// (the two sums over d are finished by lane exchanges among the LPC lanes).  The walk is a chain of dependent steps, so its time per
+// token is the latency of one step: the more lanes share a column the shorter the step (LPC = 16 at d >= 64).  q, k, g of CH tokens
+// at a time sit in LDS, rows padded so that the parts fall into different banks; the next CH tokens are fetched into registers
+// while the current ones are used.
+template <int DP, int LPC, int CH> __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaArgs p, const float* __restrict__ prep, int P) {
+    constexpr int RS = DP + 4, ROW = LPC * DP, TOT = CH * ROW, NPT = (TOT + 255) / 256, CPB = 256 / LPC;
+    __shared__ __align__(16) float sq[2][CH][LPC][RS], sk[2][CH][LPC][RS], sg[2][CH][LPC][RS];
     __shared__ float sb[2][CH], sgh[2][CH];
     const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
-    const int col = blockIdx.z * 64 + (tid >> 2), part = tid & 3;
+    const int col = blockIdx.z * CPB + tid / LPC, part = tid % LPC;
     const int d = p.d, vd = p.vd, g = h / (p.H / p.G);
     const int tb = (int)p.cu_q[s], te = (int)p.cu_q[s + 1];
     if (te <= tb) return;
@@ -771,7 +790,7 @@ template <int DP, int CH> __global__ __launch_bounds__(256) void delta_scan_kern
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int n = 0; n < NPT; ++n) {
-            const int idx = tid + n * 256, c = idx / (4 * DP), ii = idx - c * (4 * DP), t = t0 + c;
+            const int idx = tid + n * 256, c = idx / ROW, ii = idx - c * ROW, t = t0 + c;
             const bool ok_ = idx < TOT && t < te && ii < d;
             const float* row = prep + (size_t)(ok_ ? t : tb) * P;
             rq[n] = ok_ ? row[q_off + ii] : 0.f;
@@ -790,7 +809,7 @@ template <int DP, int CH> __global__ __launch_bounds__(256) void delta_scan_kern
         for (int n = 0; n < NPT; ++n) {
             const int idx = tid + n * 256;
             if (idx < TOT) {
-                const int c = idx / (4 * DP), ii = idx - c * (4 * DP), pp = ii / DP, r = ii - pp * DP;
+                const int c = idx / ROW, ii = idx - c * ROW, pp = ii / DP, r = ii - pp * DP;
                 sq[buf][c][pp][r] = rq[n]; sk[buf][c][pp][r] = rk[n]; sg[buf][c][pp][r] = rg[n];
             }
         }
@@ -819,14 +838,12 @@ template <int DP, int CH> __global__ __launch_bounds__(256) void delta_scan_kern
 #pragma unroll
                     for (int r = 0; r < DP; ++r) { S[r] *= gh; kv = fmaf(S[r], sk[buf][c][part][r], kv); }
                 }
-                kv += __shfl_xor(kv, 1);
-                kv += __shfl_xor(kv, 2);
+                kv = column_sum<LPC>(kv);
                 const float u = sb[buf][c] * (vc[c] - kv);
                 float o = 0.f;
 #pragma unroll
                 for (int r = 0; r < DP; ++r) { S[r] = fmaf(sk[buf][c][part][r], u, S[r]); o = fmaf(S[r], sq[buf][c][part][r], o); }
-                o += __shfl_xor(o, 1);
-                o += __shfl_xor(o, 2);
+                o = column_sum<LPC>(o);
                 if (own && part == 0) p.o[((size_t)(t0 + c) * p.H + h) * vd + col] = o;
             }
         }
@@ -1160,13 +1177,17 @@ int mi355_hyb_delta_rule(float* o, float* state, int64_t state_stride, const flo
     const int P = 2 * kv_heads * dim + heads * (decay_channels ? dim : 1) + heads;
     delta_prep_kernel<<<dim3(num_tokens, heads), 64, 0, s_>>>(p, scratch, P, num_tokens);
     LAUNCH_OK();
-    const dim3 grid(num_seqs, heads, (vdim + 63) / 64);
-    const int dp = (dim + 3) / 4;
-    if (dp <= 4) delta_scan_kernel<4, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
-    else if (dp <= 8) delta_scan_kernel<8, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
-    else if (dp <= 16) delta_scan_kernel<16, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
-    else if (dp <= 32) delta_scan_kernel<32, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
-    else delta_scan_kernel<64, 4><<<grid, 256, 0, s_>>>(p, scratch, P);
+    if (dim < 64) {
+        const dim3 grid(num_seqs, heads, (vdim + 63) / 64);
+        if (dim <= 16) delta_scan_kernel<4, 4, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+        else if (dim <= 32) delta_scan_kernel<8, 4, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+        else delta_scan_kernel<16, 4, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+    } else {
+        const dim3 grid(num_seqs, heads, (vdim + 15) / 16);
+        if (dim <= 64) delta_scan_kernel<4, 16, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+        else if (dim <= 128) delta_scan_kernel<8, 16, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+        else delta_scan_kernel<16, 16, 8><<<grid, 256, 0, s_>>>(p, scratch, P);
+    }
     LAUNCH_OK(); return 0;
 }
 
