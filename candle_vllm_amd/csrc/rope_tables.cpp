@@ -156,13 +156,14 @@ extern "C" int mi355_rope_tables_f64(float* cos_out, float* sin_out, int32_t rot
     double pos_div = 1.0;
     if (type == MI355_ROPE_LINEAR) { if (sc->factor <= 0) return 1; pos_div = sc->factor; }
     if (type == MI355_ROPE_LLAMA3) {
-        if (sc->factor <= 0 || sc->low_freq_factor <= 0 || sc->high_freq_factor <= 0 || sc->high_freq_factor == sc->low_freq_factor) return 1;
+        if (sc->factor <= 0 || sc->low_freq_factor <= 0 || sc->high_freq_factor <= 0) return 1;
         const double orig = original_max(sc, max_position_embeddings, max_seq_len);
         const double low_wl = orig / sc->low_freq_factor, high_wl = orig / sc->high_freq_factor;
         for (double& freq : f) {
             const double wavelen = 2.0 * M_PI / freq;
             if (wavelen < high_wl) continue;
             if (wavelen > low_wl) { freq /= sc->factor; continue; }
+            if (sc->high_freq_factor == sc->low_freq_factor) continue;     // no band between the two wavelengths
             const double smooth = (orig / wavelen - sc->low_freq_factor) / (sc->high_freq_factor - sc->low_freq_factor);
             freq = (1.0 - smooth) * freq / sc->factor + smooth * freq;
         }
