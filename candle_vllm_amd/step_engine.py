@@ -53,7 +53,8 @@ class StepEngine:
         """run the not yet cached tokens of `rids` as one batch.  want: per request, the places among its new tokens whose logits
         are asked for (default: the last).  -> logits f32 [sum of wanted places, vocab] (torch, on the device)"""
         group = [self.seqs[r] for r in rids]
-        meta = self.be.prepare_prompt(group, chunk=0)
+        pending = sum(s.get_len() - s.get_num_cached_tokens() for s in group)
+        meta = self.be.prepare_prompt(group, chunk=0, tok_cap=max(16, pending))
         cu = np.asarray(meta["cu_seqlens_q"]).astype(np.int64)
         if want is None:
             rows = (cu[1:] - 1).tolist()
