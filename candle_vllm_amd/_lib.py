@@ -341,13 +341,16 @@ class HybridLayer(ctypes.Structure):
                 ("a_rot_dims", c_i32), ("a_has_sink", c_i32), ("a_qk_norm", c_i32), ("a_scale", c_f32), ("a_out_scale", c_f32),
                 ("d_heads", c_i32), ("d_kv_heads", c_i32), ("d_dim", c_i32), ("d_vdim", c_i32), ("d_conv", c_i32),
                 ("d_decay_channels", c_i32), ("d_a_rank", c_i32), ("d_gate", c_i32), ("d_g_rank", c_i32), ("d_out_scale", c_f32),
-                ("g_width", c_i32), ("mlp_kind", c_i32), ("mlp_ff", c_i32), ("mlp_limit", c_f32), ("mlp_alpha", c_f32)]
+                ("g_width", c_i32), ("mlp_kind", c_i32), ("mlp_ff", c_i32), ("mlp_limit", c_f32), ("mlp_alpha", c_f32),
+                ("a_rot_interleaved", c_i32), ("a_kv_rank", c_i32), ("a_rot_dim", c_i32), ("a_head_gate", c_i32), ("a_conv", c_i32),
+                ("a_norm_whole", c_i32), ("a_v_unit", c_i32), ("a_softcap", c_f32), ("a_talk", c_i32), ("share_with", c_i32)]
 
 
 class HybridConfig(ctypes.Structure):
     """mirror of `mi355_hybrid_config`"""
     _fields_ = [("width", c_i32), ("vocab", c_i32), ("n_layers", c_i32), ("dtype", c_i32), ("block_size", c_i32),
-                ("state_slots", c_i32), ("norm_eps", c_f32), ("unit_eps", c_f32)]
+                ("state_slots", c_i32), ("norm_eps", c_f32), ("unit_eps", c_f32),
+                ("residual_form", c_i32), ("resid_alpha", c_f32), ("norm_groups", c_i32)]
 
 
 _sig("mi355_be_state_init", c_i32, [c_vp, c_i32])
@@ -388,6 +391,17 @@ _sig("mi355_hyb_delta_rule_scratch_floats", ctypes.c_int, [c_i32] * 5)
 _sig("mi355_hyb_gated_norm", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_i64])
 _sig("mi355_hyb_mingru", ctypes.c_int, [c_vp, c_i32, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_clamped_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_f32, c_f32, c_i64])
+_sig("mi355_hyb_window_attention_ex", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 8 + [c_i32] * 9 + [c_f32, c_f32, c_i32, c_i32, c_f32,
+                                                                                                        c_i32, c_i32, c_i64])
+_sig("mi355_hyb_head_mix", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_head_gate", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_attn_prepare_whole", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_vp] * 3 + [c_i32] * 6 + [c_f32, c_i32, c_i64])
+_sig("mi355_hyb_latent_prepare", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_i32, c_i32] + [c_vp] * 6 + [c_i32] * 7 + [c_f32, c_i32, c_i64])
+_sig("mi355_hyb_linear_batched", ctypes.c_int, [c_vp, c_i32, c_i64, c_vp, c_i32, c_i32, c_i64, c_vp, c_i64, c_i32, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_resid_norm", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_f32, c_f32, c_i64])
+_sig("mi355_hyb_gather_group_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_gelu_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_conv", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 5 + [c_i64])
 
 # the hand-written ctypes mirrors must have the layout the library was built with
 for _id, _cls in ((0, QmmDesc), (1, LlamaConfig), (2, DenseConfig), (3, RopeScaling), (4, HybridConfig), (5, HybridLayer)):

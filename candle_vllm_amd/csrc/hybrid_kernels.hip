@@ -67,16 +67,24 @@ struct LinArgs {
     const void* w; const float* bias;
     int T, N, K;
     int a_vec, w_vec;       // rows may be read 16 bytes at a time
+    int64_t a_bs, w_bs, o_bs;   // blockIdx.z = one of several independent products of this shape: element strides of its operands
 };
+template <typename TA> __device__ __forceinline__ void lin_batch(LinArgs& p) {
+    const int64_t z = blockIdx.z;
+    p.a = static_cast<const TA*>(p.a) + z * p.a_bs;
+    p.out += z * p.o_bs;
+}
+template <typename TW> __device__ __forceinline__ const TW* lin_w(const LinArgs& p) { return static_cast<const TW*>(p.w) + (int64_t)blockIdx.z * p.w_bs; }
 
 // Prompt-sized products, bf16 weights.  A workgroup of four waves owns 64 output columns (16 weight rows per wave) and 16 MT tokens;
 // fragments go from global memory / L2 straight into registers: lane (m16, kg) holds operands 8 kg .. 8 kg + 7 of row m16 of a
 // 32-wide K step on both sides, the accumulator holds tokens 4 kg + v of column m16.
 template <typename TA, int MT> __global__ __launch_bounds__(256) void linear_bf16_tile_kernel(LinArgs p) {
+    lin_batch<TA>(p);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, kg = lane >> 4;
     const int n = blockIdx.x * 64 + wave * 16 + m16;
     const int t0 = blockIdx.y * (16 * MT);
-    const uint16_t* wrow = static_cast<const uint16_t*>(p.w) + (size_t)(n < p.N ? n : 0) * p.K;
+    const uint16_t* wrow = lin_w<uint16_t>(p) + (size_t)(n < p.N ? n : 0) * p.K;
     const TA* arow[MT];
     bool aok[MT];
 #pragma unroll
@@ -119,8 +127,9 @@ __global__ __launch_bounds__(256) void linear_bf16_lds_kernel(LinArgs p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, m16 = lane & 15, kg = lane >> 4;
     const int wr = wave >> 1, wc = wave & 1;
     const int n0 = blockIdx.x * 128, t0 = blockIdx.y * 128;
+    lin_batch<uint16_t>(p);
     const uint16_t* A = static_cast<const uint16_t*>(p.a);
-    const uint16_t* W = static_cast<const uint16_t*>(p.w);
+    const uint16_t* W = lin_w<uint16_t>(p);
     // staging: thread -> rows r0 and r0 + 64 of both slices, 16-byte chunk ch of the 64-byte row
     const int r0 = tid >> 2, ch = tid & 3;
     const uint16_t* asrc[2]; const uint16_t* wsrc[2]; bool aok[2], wok[2];
@@ -189,10 +198,11 @@ __global__ __launch_bounds__(256) void linear_bf16_lds_kernel(LinArgs p) {
 // 32-wide K steps in turn (UNR steps in flight per wave) and add their partial tiles through LDS.
 template <typename TA, int NW, int UNR> __global__ __launch_bounds__(64 * NW) void linear_bf16_stream_kernel(LinArgs p) {
     __shared__ float part[NW][4][64];
+    lin_batch<TA>(p);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, kg = lane >> 4;
     const int n = blockIdx.x * 16 + m16;
     const bool nok = n < p.N, aok = m16 < p.T;
-    const uint16_t* wrow = static_cast<const uint16_t*>(p.w) + (size_t)(nok ? n : 0) * p.K;
+    const uint16_t* wrow = lin_w<uint16_t>(p) + (size_t)(nok ? n : 0) * p.K;
     const TA* arow = static_cast<const TA*>(p.a) + (size_t)(aok ? m16 : 0) * p.lda;
     f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
     for (int k0 = wave * 32 * UNR; k0 < p.K; k0 += NW * 32 * UNR) {
@@ -228,8 +238,9 @@ __global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs p) {
     __shared__ float As[16][68], Ws[16][68];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int n0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
+    lin_batch<float>(p);
     const float* A = static_cast<const float*>(p.a);
-    const float* W = static_cast<const float*>(p.w);
+    const float* W = lin_w<float>(p);
     float acc[4][4] = {};
     for (int k0 = 0; k0 < p.K; k0 += 16) {
 #pragma unroll
@@ -315,6 +326,63 @@ template <typename TO> __global__ __launch_bounds__(256) void gather_norm_kernel
     for (int i = threadIdx.x; i < width; i += blockDim.x) st<TO>(out, (size_t)r * width + i, xr[i] * inv * w[i]);
 }
 
+// x <- N(alpha x + y) w with the norm BEHIND the sum: the vector is cut into `groups` equal consecutive parts and every part is
+// divided by its own root mean square.  One workgroup per token; the sum stays in registers between the two passes (width <= 256 x 16).
+__global__ __launch_bounds__(256) void resid_norm_kernel(float* x, uint16_t* xcopy, const float* y, int ldy, const float* w, int width,
+                                                         int groups, float alpha, float eps) {
+    __shared__ float red[4];
+    __shared__ float inv_s[64];
+    const int t = blockIdx.x, part = width / groups;
+    float* xr = x + (size_t)t * width;
+    const float* yr = y + (size_t)t * ldy;
+    for (int g0 = 0; g0 < groups; g0 += 64) {
+        const int gn = min(64, groups - g0);
+        for (int g = 0; g < gn; ++g) {
+            float ss = 0.f;
+            for (int i = threadIdx.x; i < part; i += blockDim.x) {
+                const int c = (g0 + g) * part + i;
+                const float v = fmaf(alpha, xr[c], yr[c]);
+                ss = fmaf(v, v, ss);
+            }
+            ss = block_sum(ss, red);
+            if (threadIdx.x == 0) inv_s[g] = 1.f / sqrtf(ss / (float)part + eps);
+        }
+        __syncthreads();
+        for (int i = threadIdx.x; i < gn * part; i += blockDim.x) {
+            const int c = g0 * part + i;
+            const float v = fmaf(alpha, xr[c], yr[c]) * inv_s[i / part] * w[c];
+            xr[c] = v;
+            if (xcopy) xcopy[(size_t)t * width + c] = f32_to_bf16(v);
+        }
+        __syncthreads();
+    }
+}
+
+// rows[r] of x -> group RMS norm with weight -> out (dt) [n_rows, width]
+template <typename TO> __global__ __launch_bounds__(256) void gather_group_norm_kernel(TO* out, const float* x, const int32_t* rows, const float* w,
+                                                                                      int width, int groups, float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x, part = width / groups;
+    const float* xr = x + (size_t)rows[r] * width;
+    for (int g = 0; g < groups; ++g) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < part; i += blockDim.x) { const float v = xr[g * part + i]; ss = fmaf(v, v, ss); }
+        ss = block_sum(ss, red);
+        const float inv = 1.f / sqrtf(ss / (float)part + eps);
+        for (int i = threadIdx.x; i < part; i += blockDim.x) { const int c = g * part + i; st<TO>(out, (size_t)r * width + c, xr[c] * inv * w[c]); }
+    }
+}
+
+__device__ __forceinline__ float gelu_tanhf_(float z) {
+    return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+template <typename TO> __global__ void gelu_glu_kernel(TO* out, const float* gu, int64_t n, int ff) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t t = i / ff; const int j = (int)(i - t * ff);
+    st<TO>(out, (size_t)i, gelu_tanhf_(gu[t * 2 * ff + j]) * gu[t * 2 * ff + ff + j]);
+}
+
 template <typename TO> __global__ void clamped_glu_kernel(TO* out, const float* gu, int64_t n, int ff, float limit, float alpha) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
@@ -379,7 +447,11 @@ struct AttnArgs {
     const void* q; const void* k_pages; const void* v_pages;
     const uint32_t* bt; const uint32_t* ctx; const uint32_t* cu_q; const int32_t* tok_seq; const float* sink;
     int n_seqs, H, G, d, vd, bs, max_blocks, window; float scale, out_scale; int cp2, out_f32;
+    int k_ld, v_ld;         // elements per page row (all key/value heads of a token; latent attention: one row serves as both)
+    float softcap;          // > 0: score <- cap tanh(score / cap)
+    int cross;              // blockIdx.z = the key/value head whose VALUES this block sums (scores still against the head's own keys)
 };
+__device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 // 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
 template <typename TC> struct Vec16;
 template <> struct Vec16<uint16_t> {
@@ -418,6 +490,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
     const int pos = (int)p.ctx[s] - n_new + (t - (int)p.cu_q[s]);
     const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
     const int g = h / (p.H / p.G);
+    const int gv = p.cross ? (int)blockIdx.z : g, oh = p.cross ? h * p.G + gv : h;
     const TC* q = static_cast<const TC*>(p.q) + ((size_t)t * p.H + h) * p.d;
     for (int i = threadIdx.x; i < p.d; i += blockDim.x) qs[i] = ld<TC>(q, i);
     __syncthreads();
@@ -438,7 +511,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
         unsigned page_row = 0;
         if (j <= pos) {
             page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
-            const TC* kr = static_cast<const TC*>(p.k_pages) + ((size_t)page_row * p.G + g) * p.d;
+            const TC* kr = static_cast<const TC*>(p.k_pages) + (size_t)page_row * p.k_ld + g * p.d;
             float dot = 0.f;
             if (VEC && DQ > 0) {
 #pragma unroll
@@ -458,7 +531,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
             } else {
                 for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
             }
-            sc = dot * p.scale;
+            sc = cap_score(dot * p.scale, p.softcap);
         }
         const float mn = fmaxf(m, wave_max(sc));
         const float pj = (j <= pos) ? expf(sc - mn) : 0.f;
@@ -475,7 +548,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
                 const size_t pr = (size_t)__shfl(page_row, jj & 63);
                 if (jj < cnt && chunk_ok) {
                     float x[EPV];
-                    Vec16<TC>::load(static_cast<const TC*>(p.v_pages) + (pr * p.G + g) * p.vd + chunk * EPV, x);
+                    Vec16<TC>::load(static_cast<const TC*>(p.v_pages) + pr * p.v_ld + gv * p.vd + chunk * EPV, x);
 #pragma unroll
                     for (int e = 0; e < EPV; ++e) acc[e] = fmaf(pv, x[e], acc[e]);
                 }
@@ -484,7 +557,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
             for (int jj = 0; jj < cnt; ++jj) {
                 const float pv = __shfl(pj, jj);
                 const size_t pr = (size_t)__shfl(page_row, jj);
-                const TC* vr = static_cast<const TC*>(p.v_pages) + (pr * p.G + g) * p.vd;
+                const TC* vr = static_cast<const TC*>(p.v_pages) + pr * p.v_ld + gv * p.vd;
 #pragma unroll
                 for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) acc[e] = fmaf(pv, ld<TC>(vr, c), acc[e]); }
             }
@@ -509,7 +582,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
         float L = p.sink ? expf(p.sink[h] - M) : 0.f;
         float cw[NW];
         for (int w = 0; w < NW; ++w) { cw[w] = pm[w] == -INFINITY ? 0.f : expf(pm[w] - M); L += pl[w] * cw[w]; }
-        const size_t base = (size_t)t * p.ldo + p.out_off + (size_t)h * p.vd;
+        const size_t base = (size_t)t * p.ldo + p.out_off + (size_t)oh * p.vd;
         for (int col = lane; col < p.vd; col += 64) {
             float o = 0.f;
             for (int w = 0; w < NW; ++w) o += pacc[w * p.vd + col] * cw[w];
@@ -541,6 +614,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
     const int t0 = (int)p.cu_q[s] + b * 16, nq = min(16, (int)p.cu_q[s + 1] - t0);
     const int pos0 = (int)p.ctx[s] - n_new + b * 16;
     const int h = blockIdx.y, g = h / (p.H / p.G), d = p.d, vd = p.vd;
+    const int gv = p.cross ? (int)blockIdx.z : g, oh = p.cross ? h * p.G + gv : h;
     const uint16_t* Q = static_cast<const uint16_t*>(p.q);
     const uint16_t* K = static_cast<const uint16_t*>(p.k_pages);
     const uint16_t* V = static_cast<const uint16_t*>(p.v_pages);
@@ -565,7 +639,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
             const int key = j0 + kt * 16 + m16;
             const bool kv = key <= hi;
             const size_t pr = kv ? (size_t)bt[key / p.bs] * p.bs + (key % p.bs) : 0;
-            const uint16_t* kr = K + (pr * p.G + g) * d + 8 * kg;
+            const uint16_t* kr = K + pr * p.k_ld + g * d + 8 * kg;
 #pragma unroll
             for (int ks = 0; ks < DK; ++ks) {
                 const uint4 kf = kv ? *reinterpret_cast<const uint4*>(kr + ks * 32) : uint4{0, 0, 0, 0};
@@ -577,7 +651,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
             const int key = j0 + lane;
             const bool kv = key <= hi;
             const size_t pr = kv ? (size_t)bt[key / p.bs] * p.bs + (key % p.bs) : 0;
-            const uint16_t* vr = V + (pr * p.G + g) * vd;
+            const uint16_t* vr = V + pr * p.v_ld + gv * vd;
 #pragma unroll
             for (int c8 = 0; c8 < VT * 2; ++c8) {
                 const uint4 x = kv ? *reinterpret_cast<const uint4*>(vr + c8 * 8) : uint4{0, 0, 0, 0};
@@ -599,7 +673,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
             for (int kt = 0; kt < 4; ++kt) {
                 const int key = j0 + kt * 16 + m16;
                 const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window);
-                sc[v][kt] = ok_ ? sacc[kt][v] * p.scale : -INFINITY;
+                sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) : -INFINITY;
                 mx[v] = fmaxf(mx[v], sc[v][kt]);
             }
 #pragma unroll
@@ -648,7 +722,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
         const float cm = expf(mrow[v] - M);
         const float L = lrow[v] * cm + (p.sink ? expf(sink - M) : 0.f);
         const float f = cm / L * p.out_scale;
-        const size_t base = (size_t)(t0 + r) * p.ldo + p.out_off + (size_t)h * vd;
+        const size_t base = (size_t)(t0 + r) * p.ldo + p.out_off + (size_t)oh * vd;
 #pragma unroll
         for (int c = 0; c < VT; ++c) {
             const float o = acc[c][v] * f;
@@ -662,6 +736,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
 struct ConvArgs {
     float* out; const float* proj; int ldp, off; const float* w; float* state; int64_t state_stride;
     const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots; const int32_t* tok_seq; int C, taps, T;
+    int act;                // 0 = none, 1 = silu
 };
 __global__ void conv_silu_kernel(ConvArgs p) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -682,7 +757,7 @@ __global__ void conv_silu_kernel(ConvArgs p) {
         }
         acc = fmaf(p.w[(size_t)c * p.taps + i], v, acc);
     }
-    p.out[idx] = siluf_(acc);
+    p.out[idx] = p.act ? siluf_(acc) : acc;
 }
 // state[j], j = 0 .. taps-2 (oldest first) <- the taps - 1 inputs that end with the portion's last token
 __global__ void conv_state_update_kernel(ConvArgs p, int n_seqs) {
@@ -972,6 +1047,107 @@ __global__ void fill_f32_kernel(float* out, float v, int64_t n) {
     if (i < n) out[i] = v;
 }
 
+// ------------------------------------------------------------------------------------------------------------ more attention glue
+struct WholePrepArgs {
+    void* q_out; void* k_pages; void* v_pages;
+    const float* src; int ld, q_off, k_off, v_off;
+    const float* qw; const float* kw; const int64_t* slots;
+    int H, G, d, vd, v_unit; float eps;
+};
+// One workgroup per token.  q and k: ONE RMS norm over the whole row part (all heads at once), weights of that size; v: every head
+// divided by its own root mean square (no weight).  q -> q_out, k and v -> the token's page row.  No rotation.
+template <typename TC> __global__ __launch_bounds__(256) void attn_prepare_whole_kernel(WholePrepArgs p) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* row = p.src + (size_t)t * p.ld;
+    const int nq = p.H * p.d, nk = p.G * p.d;
+    const int64_t slot = p.slots[t];
+    float sq = 0.f, sk = 0.f;
+    if (p.qw) for (int i = threadIdx.x; i < nq; i += blockDim.x) { const float v = row[p.q_off + i]; sq = fmaf(v, v, sq); }
+    if (p.kw) for (int i = threadIdx.x; i < nk; i += blockDim.x) { const float v = row[p.k_off + i]; sk = fmaf(v, v, sk); }
+    sq = block_sum(sq, red);
+    sk = block_sum(sk, red);
+    const float iq = p.qw ? 1.f / sqrtf(sq / (float)nq + p.eps) : 1.f, ik = p.kw ? 1.f / sqrtf(sk / (float)nk + p.eps) : 1.f;
+    TC* qd = static_cast<TC*>(p.q_out) + (size_t)t * nq;
+    for (int i = threadIdx.x; i < nq; i += blockDim.x) st<TC>(qd, i, row[p.q_off + i] * iq * (p.qw ? p.qw[i] : 1.f));
+    if (slot < 0) return;
+    TC* kd = static_cast<TC*>(p.k_pages) + (size_t)slot * nk;
+    for (int i = threadIdx.x; i < nk; i += blockDim.x) st<TC>(kd, i, row[p.k_off + i] * ik * (p.kw ? p.kw[i] : 1.f));
+    TC* vdst = static_cast<TC*>(p.v_pages) + (size_t)slot * p.G * p.vd;
+    for (int g = wave; g < p.G; g += (int)(blockDim.x >> 6)) {          // a wave per value head
+        const float* vr = row + p.v_off + g * p.vd;
+        float ss = 0.f;
+        if (p.v_unit) { for (int i = lane; i < p.vd; i += 64) ss = fmaf(vr[i], vr[i], ss); ss = wave_sum(ss); }
+        const float iv = p.v_unit ? 1.f / sqrtf(ss / (float)p.vd + p.eps) : 1.f;
+        for (int i = lane; i < p.vd; i += 64) st<TC>(vdst, (size_t)g * p.vd + i, vr[i] * iv);
+    }
+}
+
+struct LatentPrepArgs {
+    void* q_out; void* pages;
+    const float* proj; int ldp, q_off, c_off;
+    const float* q_abs; const float* cw; const float* cos_t; const float* sin_t;
+    const int64_t* positions; const int64_t* slots;
+    int H, d, r, rank, rot, interleaved; float eps;
+};
+// element i of a rot_dim-wide vector v after the rotation of its first `rot` dimensions by the angles of position `pos`
+__device__ __forceinline__ float rotated_elem(const float* v, int i, int rot, int interleaved, const float* cs, const float* sn) {
+    if (i >= rot) return v[i];
+    const int half = rot / 2;
+    if (interleaved) {
+        const int pr = i >> 1;
+        return (i & 1) ? v[i] * cs[pr] + v[i - 1] * sn[pr] : v[i] * cs[pr] - v[i + 1] * sn[pr];
+    }
+    return i < half ? v[i] * cs[i] - v[i + half] * sn[i] : v[i] * cs[i - half] + v[i - half] * sn[i - half];
+}
+// One workgroup per token: the latent's RMS norm and the rotation of the shared key part -> the token's page row [latent | key part];
+// per head [absorbed query (already multiplied by the key up-projection) | rotated query part] -> q_out.
+template <typename TC> __global__ __launch_bounds__(256) void latent_prepare_kernel(LatentPrepArgs p) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, dq = p.rank + p.r;
+    const float* row = p.proj + (size_t)t * p.ldp;
+    const int64_t pos = p.positions[t], slot = p.slots[t];
+    const float* cs = p.cos_t + pos * (p.rot / 2);
+    const float* sn = p.sin_t + pos * (p.rot / 2);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < p.rank; i += blockDim.x) { const float v = row[p.c_off + i]; ss = fmaf(v, v, ss); }
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)p.rank + p.eps);
+    if (slot >= 0) {
+        TC* dst = static_cast<TC*>(p.pages) + (size_t)slot * dq;
+        for (int i = threadIdx.x; i < p.rank; i += blockDim.x) st<TC>(dst, i, row[p.c_off + i] * inv * p.cw[i]);
+        const float* kr = row + p.c_off + p.rank;
+        for (int i = threadIdx.x; i < p.r; i += blockDim.x) st<TC>(dst, p.rank + i, rotated_elem(kr, i, p.rot, p.interleaved, cs, sn));
+    }
+    TC* qd = static_cast<TC*>(p.q_out) + (size_t)t * p.H * dq;
+    for (int i = threadIdx.x; i < p.H * dq; i += blockDim.x) {
+        const int h = i / dq, c = i - h * dq;
+        const float v = c < p.rank ? p.q_abs[((size_t)t * p.H + h) * p.rank + c]
+                                   : rotated_elem(row + p.q_off + h * (p.d + p.r) + p.d, c - p.rank, p.rot, p.interleaved, cs, sn);
+        st<TC>(qd, i, v);
+    }
+}
+
+// out[t, h, :] = sum_g talk[h, g] a[t, g, kv head of h, :]
+template <typename TO> __global__ void head_mix_kernel(TO* out, const float* a, const float* talk, int64_t n, int H, int G, int vd) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t t = i / ((int64_t)H * vd);
+    const int rem = (int)(i - t * H * vd), h = rem / vd, c = rem - h * vd, kv = h / (H / G);
+    const float* at = a + (size_t)t * H * G * vd + (size_t)kv * vd + c;
+    float acc = 0.f;
+    for (int g = 0; g < H; ++g) acc = fmaf(talk[h * H + g], at[(size_t)g * G * vd], acc);
+    st<TO>(out, (size_t)i, acc);
+}
+
+template <typename TO> __global__ void head_gate_kernel(TO* out, const float* in, const float* gate_in, int ldg, int64_t n, int H, int vd) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t t = i / ((int64_t)H * vd);
+    const int h = (int)(i - t * H * vd) / vd;
+    st<TO>(out, (size_t)i, gate_in ? in[i] * sigmoidf_(gate_in[(size_t)t * ldg + h]) : in[i]);
+}
+
 int g_attn_mfma = 1;            // mi355_hyb_set_attention_mfma(0): prompt steps take the generic kernel too (A/B, tests of both paths)
 
 #define LAUNCH_OK() do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)
@@ -1004,35 +1180,46 @@ int mi355_hyb_fill_f32(float* out, float v, int64_t n, int64_t stream) {
     LAUNCH_OK(); return 0;
 }
 
-int mi355_hyb_linear(float* out, int32_t ldo, const void* a, int32_t a_dtype, int32_t lda, const void* w, const float* bias,
-                     int32_t T, int32_t n, int32_t k, int32_t dtype, int64_t stream) {
-    if (!out || !a || !w || T < 0 || n <= 0 || k <= 0 || ldo < n || lda < k || !is_dt(dtype) || !is_dt(a_dtype)) return -1;
+static int linear_launch(float* out, int32_t ldo, int64_t o_bs, const void* a, int32_t a_dtype, int32_t lda, int64_t a_bs, const void* w,
+                         int64_t w_bs, const float* bias, int32_t T, int32_t n, int32_t k, int32_t batch, int32_t dtype, int64_t stream) {
+    if (!out || !a || !w || T < 0 || n <= 0 || k <= 0 || ldo < n || lda < k || batch <= 0 || batch > 65535 || !is_dt(dtype) || !is_dt(a_dtype)) return -1;
     if (T == 0) return 0;
-    LinArgs p{out, ldo, a, lda, w, bias, T, n, k, 0, 0};
+    LinArgs p{out, ldo, a, lda, w, bias, T, n, k, 0, 0, a_bs, w_bs, o_bs};
     hipStream_t st_ = to_stream(stream);
+    const unsigned nz = (unsigned)batch;
     if (dtype == MI355_DTYPE_F32) {
         if (a_dtype != MI355_DTYPE_F32) return -1;
-        linear_f32_kernel<<<dim3((n + 63) / 64, (T + 63) / 64), 256, 0, st_>>>(p);
+        linear_f32_kernel<<<dim3((n + 63) / 64, (T + 63) / 64, nz), 256, 0, st_>>>(p);
         LAUNCH_OK(); return 0;
     }
     const int a_bytes = a_dtype == MI355_DTYPE_F32 ? 4 : 2;
-    p.w_vec = (k % 8 == 0) && ((uintptr_t)w % 16 == 0);
-    p.a_vec = ((size_t)lda * a_bytes % 16 == 0) && ((uintptr_t)a % 16 == 0);
+    p.w_vec = (k % 8 == 0) && ((uintptr_t)w % 16 == 0) && (w_bs % 8 == 0);
+    p.a_vec = ((size_t)lda * a_bytes % 16 == 0) && ((uintptr_t)a % 16 == 0) && ((size_t)a_bs * a_bytes % 16 == 0);
     const bool af = a_dtype == MI355_DTYPE_F32;
     if (T <= 16) {
-        const dim3 grid((n + 15) / 16);
+        const dim3 grid((n + 15) / 16, 1, nz);
         if (k >= 2048) { if (af) linear_bf16_stream_kernel<float, 4, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 4, 4><<<grid, 256, 0, st_>>>(p); }
         else { if (af) linear_bf16_stream_kernel<float, 2, 2><<<grid, 128, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 2, 2><<<grid, 128, 0, st_>>>(p); }
     } else if (T > 32 && !af && p.a_vec && p.w_vec && k % 32 == 0) {
-        linear_bf16_lds_kernel<<<dim3((n + 127) / 128, (T + 127) / 128), 256, 0, st_>>>(p);
+        linear_bf16_lds_kernel<<<dim3((n + 127) / 128, (T + 127) / 128, nz), 256, 0, st_>>>(p);
     } else if (T <= 32) {
-        const dim3 grid((n + 63) / 64, (T + 31) / 32);
+        const dim3 grid((n + 63) / 64, (T + 31) / 32, nz);
         if (af) linear_bf16_tile_kernel<float, 2><<<grid, 256, 0, st_>>>(p); else linear_bf16_tile_kernel<uint16_t, 2><<<grid, 256, 0, st_>>>(p);
     } else {
-        const dim3 grid((n + 63) / 64, (T + 63) / 64);
+        const dim3 grid((n + 63) / 64, (T + 63) / 64, nz);
         if (af) linear_bf16_tile_kernel<float, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_tile_kernel<uint16_t, 4><<<grid, 256, 0, st_>>>(p);
     }
     LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_linear(float* out, int32_t ldo, const void* a, int32_t a_dtype, int32_t lda, const void* w, const float* bias,
+                     int32_t T, int32_t n, int32_t k, int32_t dtype, int64_t stream) {
+    return linear_launch(out, ldo, 0, a, a_dtype, lda, 0, w, 0, bias, T, n, k, 1, dtype, stream);
+}
+int mi355_hyb_linear_batched(float* out, int32_t ldo, int64_t o_bs, const void* a, int32_t a_dtype, int32_t lda, int64_t a_bs,
+                             const void* w, int64_t w_bs, int32_t T, int32_t n, int32_t k, int32_t batch, int32_t dtype, int64_t stream) {
+    if (o_bs < 0 || a_bs < 0 || w_bs < 0) return -1;
+    return linear_launch(out, ldo, o_bs, a, a_dtype, lda, a_bs, w, w_bs, nullptr, T, n, k, batch, dtype, stream);
 }
 
 int mi355_hyb_embed(float* x, void* xcopy, const void* table, const uint32_t* ids, int32_t T, int32_t width, int32_t vocab, int32_t dtype,
@@ -1092,23 +1279,40 @@ int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
                                    const uint32_t* cu_seqlens_q, const int32_t* tok_seq, const float* sink, int32_t num_seqs,
                                    int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
                                    int32_t max_blocks, int32_t window, float scale, float out_scale, int32_t dtype, int64_t stream) {
+    return mi355_hyb_window_attention_ex(out, out_dtype, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq,
+                                         sink, num_seqs, T, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale,
+                                         0, 0, 0.f, 0, dtype, stream);
+}
+
+int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                                   const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                                   const uint32_t* cu_seqlens_q, const int32_t* tok_seq, const float* sink, int32_t num_seqs,
+                                   int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
+                                   int32_t max_blocks, int32_t window, float scale, float out_scale, int32_t k_ld, int32_t v_ld,
+                                   float softcap, int32_t cross_values, int32_t dtype, int64_t stream) {
     if (!out || !q || !k_pages || !v_pages || !block_tables || !context_lens || !cu_seqlens_q || !tok_seq) return -1;
     if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return -1;
-    if (block_size <= 0 || max_blocks <= 0 || window < 0) return -1;
+    if (block_size <= 0 || max_blocks <= 0 || window < 0 || softcap < 0.f) return -1;
+    if (k_ld == 0) k_ld = kv_heads * dim;
+    if (v_ld == 0) v_ld = kv_heads * vdim;
+    if (k_ld < kv_heads * dim || v_ld < kv_heads * vdim) return -1;
     if (T <= 0) return 0;
     const bool f = dtype == MI355_DTYPE_F32;
+    const int cross = cross_values ? 1 : 0, nz = cross ? kv_heads : 1;
     AttnArgs p{out, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq, sink,
-               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale, 64, out_dtype == MI355_DTYPE_F32};
-    const dim3 grid(T, heads);
+               num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale, 64, out_dtype == MI355_DTYPE_F32,
+               k_ld, v_ld, softcap, cross};
+    const dim3 grid(T, heads, nz);
     hipStream_t s_ = to_stream(stream);
     const int epv = f ? 4 : 8;
-    const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0;
+    const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 &&
+                     k_ld % epv == 0 && v_ld % epv == 0;
     if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; }
     else if (vdim > 512) return -1;
     // prompt-sized steps over bf16 pages: the matrix-core kernel (a tile of 16 tokens never spans two sequences)
     if (!f && T >= 64 && dim % 32 == 0 && dim <= 256 && vdim % 16 == 0 && vdim <= 256 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
-        (uintptr_t)v_pages % 16 == 0 && g_attn_mfma) {
-        const dim3 mgrid((T + 15) / 16 + num_seqs, heads);
+        (uintptr_t)v_pages % 16 == 0 && k_ld % 8 == 0 && v_ld % 8 == 0 && g_attn_mfma) {
+        const dim3 mgrid((T + 15) / 16 + num_seqs, heads, nz);
         const int dk = dim / 32, vt = vdim / 16;
 #define WM(DK, VT) window_attention_mfma_kernel<DK, VT><<<mgrid, 64, 0, s_>>>(p)
 #define WMV(DK) do { if (vt <= 2) { if (vt == 1) WM(DK, 1); else WM(DK, 2); } else if (vt <= 4) { if (vt == 3) WM(DK, 3); else WM(DK, 4); } \
@@ -1139,10 +1343,18 @@ int mi355_hyb_conv_silu(float* out, const float* proj, int32_t ldp, int32_t off,
                             int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
                             const int32_t* state_slots, const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t channels,
                             int32_t taps, int64_t stream) {
+    return mi355_hyb_conv(out, proj, ldp, off, w, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, num_seqs, T,
+                          channels, taps, 1, stream);
+}
+
+int mi355_hyb_conv(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* conv_state,
+                   int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                   const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t channels, int32_t taps, int32_t act, int64_t stream) {
+    if (act != 0 && act != 1) return -1;
     if (!out || !proj || !w || !conv_state || !context_lens || !cu_seqlens_q || !state_slots || !tok_seq) return -1;
     if (channels <= 0 || taps < 1 || taps > 16) return -1;
     if (T <= 0) return 0;
-    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T};
+    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T, act};
     const int64_t n = (int64_t)T * channels;
     conv_silu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(p);
     LAUNCH_OK(); return 0;
@@ -1153,7 +1365,7 @@ int mi355_hyb_conv_state_update(float* conv_state, int64_t state_stride, const f
                                 int32_t num_seqs, int32_t channels, int32_t taps, int64_t stream) {
     if (!conv_state || !proj || !context_lens || !cu_seqlens_q || !state_slots || channels <= 0 || taps < 1 || taps > 16) return -1;
     if (num_seqs <= 0 || taps == 1) return 0;
-    ConvArgs p{nullptr, proj, ldp, off, nullptr, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, nullptr, channels, taps, 0};
+    ConvArgs p{nullptr, proj, ldp, off, nullptr, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, nullptr, channels, taps, 0, 0};
     const int n = num_seqs * channels;
     conv_state_update_kernel<<<(n + 255) / 256, 256, 0, to_stream(stream)>>>(p, num_seqs);
     LAUNCH_OK(); return 0;
@@ -1216,6 +1428,86 @@ int mi355_hyb_mingru(void* out, int32_t out_dtype, float* state, int64_t state_s
     }
     if (out_dtype == MI355_DTYPE_F32) mingru_kernel<float, 8><<<grid, 64, 0, to_stream(stream)>>>(p);
     else mingru_kernel<uint16_t, 8><<<grid, 64, 0, to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_resid_norm(float* x, void* xcopy, const float* y, int32_t ldy, const float* w, int32_t T, int32_t width, int32_t groups,
+                         float alpha, float eps, int64_t stream) {
+    if (groups <= 0) groups = 1;
+    if (!x || !y || !w || width <= 0 || ldy < width || width % groups) return -1;
+    if (T <= 0) return 0;
+    resid_norm_kernel<<<T, 256, 0, to_stream(stream)>>>(x, (uint16_t*)xcopy, y, ldy, w, width, groups, alpha, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_gather_group_norm(void* out, int32_t out_dtype, const float* x, const int32_t* rows, const float* w, int32_t n_rows,
+                                int32_t width, int32_t groups, float eps, int64_t stream) {
+    if (groups <= 0) groups = 1;
+    if (!out || !x || !rows || !w || !is_dt(out_dtype) || width <= 0 || width % groups) return -1;
+    if (n_rows <= 0) return 0;
+    if (out_dtype == MI355_DTYPE_F32) gather_group_norm_kernel<float><<<n_rows, 256, 0, to_stream(stream)>>>((float*)out, x, rows, w, width, groups, eps);
+    else gather_group_norm_kernel<uint16_t><<<n_rows, 256, 0, to_stream(stream)>>>((uint16_t*)out, x, rows, w, width, groups, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_gelu_glu(void* out, int32_t out_dtype, const float* gu, int32_t T, int32_t ff, int64_t stream) {
+    if (!out || !gu || ff <= 0 || !is_dt(out_dtype)) return -1;
+    const int64_t n = (int64_t)T * ff;
+    if (n <= 0) return 0;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (out_dtype == MI355_DTYPE_F32) gelu_glu_kernel<float><<<grid, 256, 0, to_stream(stream)>>>((float*)out, gu, n, ff);
+    else gelu_glu_kernel<uint16_t><<<grid, 256, 0, to_stream(stream)>>>((uint16_t*)out, gu, n, ff);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_attn_prepare_whole(void* q_out, void* k_pages, void* v_pages, const float* src, int32_t ld, int32_t q_off, int32_t k_off,
+                                 int32_t v_off, const float* q_norm_w, const float* k_norm_w, const int64_t* slot_mapping, int32_t T,
+                                 int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t v_unit, float eps, int32_t dtype,
+                                 int64_t stream) {
+    if (!q_out || !k_pages || !v_pages || !src || !slot_mapping || !is_dt(dtype)) return -1;
+    if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return -1;
+    if (T <= 0) return 0;
+    WholePrepArgs p{q_out, k_pages, v_pages, src, ld, q_off, k_off, v_off, q_norm_w, k_norm_w, slot_mapping, heads, kv_heads, dim, vdim,
+                    v_unit ? 1 : 0, eps};
+    if (dtype == MI355_DTYPE_F32) attn_prepare_whole_kernel<float><<<T, 256, 0, to_stream(stream)>>>(p);
+    else attn_prepare_whole_kernel<uint16_t><<<T, 256, 0, to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_latent_prepare(void* q_out, void* pages, const float* proj, int32_t ldp, int32_t q_off, int32_t c_off, const float* q_abs,
+                             const float* c_norm_w, const float* cos_t, const float* sin_t, const int64_t* positions,
+                             const int64_t* slot_mapping, int32_t T, int32_t heads, int32_t dim, int32_t rot_dim, int32_t kv_rank,
+                             int32_t rot_dims, int32_t interleaved, float eps, int32_t dtype, int64_t stream) {
+    if (!q_out || !pages || !proj || !q_abs || !c_norm_w || !positions || !slot_mapping || !is_dt(dtype)) return -1;
+    if (heads <= 0 || dim <= 0 || rot_dim < 0 || kv_rank <= 0 || rot_dims < 0 || rot_dims > rot_dim || (rot_dims & 1)) return -1;
+    if (rot_dims > 0 && (!cos_t || !sin_t)) return -1;
+    if (T <= 0) return 0;
+    LatentPrepArgs p{q_out, pages, proj, ldp, q_off, c_off, q_abs, c_norm_w, cos_t, sin_t, positions, slot_mapping,
+                     heads, dim, rot_dim, kv_rank, rot_dims, interleaved ? 1 : 0, eps};
+    if (dtype == MI355_DTYPE_F32) latent_prepare_kernel<float><<<T, 256, 0, to_stream(stream)>>>(p);
+    else latent_prepare_kernel<uint16_t><<<T, 256, 0, to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_head_mix(void* out, int32_t out_dtype, const float* a, const float* talk, int32_t T, int32_t heads, int32_t kv_heads,
+                       int32_t vdim, int64_t stream) {
+    if (!out || !a || !talk || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || vdim <= 0) return -1;
+    const int64_t n = (int64_t)T * heads * vdim;
+    if (n <= 0) return 0;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (out_dtype == MI355_DTYPE_F32) head_mix_kernel<float><<<grid, 256, 0, to_stream(stream)>>>((float*)out, a, talk, n, heads, kv_heads, vdim);
+    else head_mix_kernel<uint16_t><<<grid, 256, 0, to_stream(stream)>>>((uint16_t*)out, a, talk, n, heads, kv_heads, vdim);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_head_gate(void* out, int32_t out_dtype, const float* in, const float* gate_in, int32_t ldg, int32_t T, int32_t heads,
+                        int32_t vdim, int64_t stream) {
+    if (!out || !in || !is_dt(out_dtype) || heads <= 0 || vdim <= 0 || (gate_in && ldg < heads)) return -1;
+    const int64_t n = (int64_t)T * heads * vdim;
+    if (n <= 0) return 0;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (out_dtype == MI355_DTYPE_F32) head_gate_kernel<float><<<grid, 256, 0, to_stream(stream)>>>((float*)out, in, gate_in, ldg, n, heads, vdim);
+    else head_gate_kernel<uint16_t><<<grid, 256, 0, to_stream(stream)>>>((uint16_t*)out, in, gate_in, ldg, n, heads, vdim);
     LAUNCH_OK(); return 0;
 }
 

@@ -1,6 +1,8 @@
 // Host layer of the layer-list ("hybrid") models (include/mi355_hybrid.h): a model is a list of layers, each with one token mixer
-// (sliding-window attention with a sink, gated delta rule, minGRU, or attention and delta rule side by side) and an optional
-// feed-forward; x <- x + norm(mixer(x)), x <- x + norm(ff(x)), the sublayers read x itself.  Like the llama-family host layers
+// (sliding-window attention with a sink, gated delta rule, minGRU, attention and delta rule side by side, latent attention, or
+// attention behind a short convolution with mixed head weights) and an optional feed-forward; x <- x + norm(mixer(x)),
+// x <- x + norm(ff(x)) -- or, with residual_form 1, x <- norm(alpha x + mixer(x)), x <- norm(alpha x + ff(x)) -- the sublayers read
+// x itself.  A layer may run on another layer's weights (share_with) and still owns its pages and state.  Like the llama-family host layers
 // (host_model.cpp, dense_model.cpp) it owns the weights, the K/V pages and the activation buffers and enqueues one step on a
 // stream; unlike them it owns a pool of recurrent state (one slot per live sequence, handed out by the block engine) and runs
 // prompts, portions of prompts and decoded tokens through the same launches.
@@ -46,7 +48,15 @@ struct HLayer {
     int64_t conv_off = 0, state_off = 0;          // floats from the start of a slot
     bool has_attn() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION; }
     bool has_delta() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA; }
+    bool is_latent() const { return c.mixer == MI355_HYB_MIX_LATENT; }
+    bool is_conv_attn() const { return c.mixer == MI355_HYB_MIX_CONV_ATTENTION; }
+    bool uses_pages() const { return has_attn() || is_latent() || is_conv_attn(); }
+    bool rotates() const { return (has_attn() || is_latent()) && c.a_rot_dims > 0; }
     int conv_channels() const { return 2 * c.d_kv_heads * c.d_dim + c.d_heads * c.d_vdim; }
+    int a_conv_channels() const { return (c.a_heads + c.a_kv_heads) * c.a_dim + c.a_kv_heads * c.a_vdim; }
+    // elements of a token's row in the key / value pages (latent attention: one row [latent | rotated key part], no value pages)
+    int k_row() const { return is_latent() ? c.a_kv_rank + c.a_rot_dim : c.a_kv_heads * c.a_dim; }
+    int v_row() const { return is_latent() ? 0 : c.a_kv_heads * c.a_vdim; }
 };
 
 struct HModel {
@@ -59,9 +69,9 @@ struct HModel {
     // activations (grow-only)
     int cap_t = 0, cap_out = 0;
     float *prep = nullptr, *x = nullptr, *proj = nullptr, *aux1 = nullptr, *aux2 = nullptr, *conv = nullptr, *o = nullptr, *y = nullptr, *gu = nullptr;
-    void *xcopy = nullptr, *q = nullptr, *mix = nullptr, *act = nullptr, *xn = nullptr;
+    void *xcopy = nullptr, *q = nullptr, *mix = nullptr, *act = nullptr, *xn = nullptr, *att = nullptr;
     int32_t* tok_seq = nullptr;
-    int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0, max_prep = 0;
+    int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0, max_prep = 0, max_att = 0;
     // captured steps (mi355_hybrid_forward_graph): one hipGraph per (device input pointers, counts); whatever re-allocates a buffer a
     // step touches drops them all
     struct StepGraph { hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; };
@@ -86,7 +96,13 @@ int in_proj_parts(const mi355_hybrid_layer& c, int32_t* off) {
         off[0] = 0; off[1] = c.g_width; off[2] = 2 * c.g_width;
         return 3 * c.g_width;
     }
-    if (c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION) {
+    if (c.mixer == MI355_HYB_MIX_LATENT) {
+        off[P_AQ] = r; r += c.a_heads * (c.a_dim + c.a_rot_dim);
+        off[P_AK] = r; r += c.a_kv_rank + c.a_rot_dim;
+        if (c.a_head_gate) { off[P_G] = r; r += c.a_heads; }
+        return r;
+    }
+    if (c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION || c.mixer == MI355_HYB_MIX_CONV_ATTENTION) {
         off[P_AQ] = r; r += c.a_heads * c.a_dim;
         off[P_AK] = r; r += c.a_kv_heads * c.a_dim;
         off[P_AV] = r; r += c.a_kv_heads * c.a_vdim;
@@ -105,7 +121,16 @@ int in_proj_parts(const mi355_hybrid_layer& c, int32_t* off) {
 bool layer_ok(const mi355_hybrid_layer& c) {
     const bool attn = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION;
     const bool delta = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA;
-    if (c.mixer < 0 || c.mixer > MI355_HYB_MIX_ATTENTION) return false;
+    if (c.mixer < 0 || c.mixer > MI355_HYB_MIX_CONV_ATTENTION || c.share_with < 0) return false;
+    if (c.mixer == MI355_HYB_MIX_LATENT) {
+        if (c.a_heads <= 0 || c.a_dim <= 0 || c.a_vdim <= 0 || c.a_kv_rank <= 0 || c.a_rot_dim < 0 || c.a_window < 0) return false;
+        if (c.a_rot_dims < 0 || c.a_rot_dims > c.a_rot_dim || (c.a_rot_dims & 1) || c.a_softcap < 0.f) return false;
+    }
+    if (c.mixer == MI355_HYB_MIX_CONV_ATTENTION) {
+        if (c.a_heads <= 0 || c.a_kv_heads <= 0 || c.a_heads % c.a_kv_heads || c.a_dim <= 0 || c.a_vdim <= 0 || c.a_window < 0) return false;
+        if (c.a_conv < 1 || c.a_conv > 16 || c.a_softcap < 0.f || c.a_rot_dims != 0) return false;
+        if (c.a_qk_norm && !c.a_norm_whole) return false;
+    }
     if (attn) {
         if (c.a_heads <= 0 || c.a_kv_heads <= 0 || c.a_heads % c.a_kv_heads || c.a_dim <= 0 || c.a_vdim <= 0 || c.a_vdim > 512) return false;
         if (c.a_window < 0 || c.a_rot_dims < 0 || c.a_rot_dims > c.a_dim || (c.a_rot_dims & 1)) return false;
@@ -118,7 +143,7 @@ bool layer_ok(const mi355_hybrid_layer& c) {
         if (c.d_gate != MI355_HYB_GATE_SIGMOID_LR && c.d_gate != MI355_HYB_GATE_SILU) return false;
     }
     if (c.mixer == MI355_HYB_MIX_MINGRU && c.g_width <= 0) return false;
-    if (c.mlp_kind < 0 || c.mlp_kind > 1 || (c.mlp_kind == 1 && c.mlp_ff <= 0)) return false;
+    if (c.mlp_kind < 0 || c.mlp_kind > 2 || (c.mlp_kind && c.mlp_ff <= 0)) return false;
     return true;
 }
 
@@ -126,7 +151,7 @@ bool layer_ok(const mi355_hybrid_layer& c) {
 bool is_matrix(int which) {
     switch (which) {
         case MI355_HW_EMBED: case MI355_HW_HEAD: case MI355_HW_IN_PROJ: case MI355_HW_OUT_PROJ: case MI355_HW_D_A2: case MI355_HW_D_G2:
-        case MI355_HW_MLP_GATE_UP: case MI355_HW_MLP_DOWN: return true;
+        case MI355_HW_MLP_GATE_UP: case MI355_HW_MLP_DOWN: case MI355_HW_L_UKT: case MI355_HW_L_UV: return true;
         default: return false;
     }
 }
@@ -140,14 +165,23 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
     }
     const HLayer& L = m->layers[layer];
     const mi355_hybrid_layer& c = L.c;
+    if (c.share_with) return -1;                               // a layer that runs on another layer's weights holds none
     switch (which) {
         case MI355_HW_NORM1: return W;
         case MI355_HW_NORM2: return c.mlp_kind ? W : -1;
         case MI355_HW_IN_PROJ: return (int64_t)L.in_rows * W;
         case MI355_HW_IN_BIAS: return L.in_rows;
         case MI355_HW_OUT_PROJ: return (int64_t)W * L.out_k;
-        case MI355_HW_A_QNORM: case MI355_HW_A_KNORM: return L.has_attn() && c.a_qk_norm ? c.a_dim : -1;
-        case MI355_HW_A_SINK: return L.has_attn() && c.a_has_sink ? c.a_heads : -1;
+        case MI355_HW_A_QNORM: if (L.is_conv_attn()) return c.a_qk_norm ? c.a_heads * c.a_dim : -1;
+                               return L.has_attn() && c.a_qk_norm ? c.a_dim : -1;
+        case MI355_HW_A_KNORM: if (L.is_conv_attn()) return c.a_qk_norm ? c.a_kv_heads * c.a_dim : -1;
+                               return L.has_attn() && c.a_qk_norm ? c.a_dim : -1;
+        case MI355_HW_A_SINK: return (L.has_attn() || L.is_latent()) && c.a_has_sink ? c.a_heads : -1;
+        case MI355_HW_A_CONV: return L.is_conv_attn() ? (int64_t)L.a_conv_channels() * c.a_conv : -1;
+        case MI355_HW_A_TALK: return L.is_conv_attn() && c.a_talk ? c.a_heads * c.a_heads : -1;
+        case MI355_HW_L_UKT: return L.is_latent() ? (int64_t)c.a_heads * c.a_kv_rank * c.a_dim : -1;
+        case MI355_HW_L_UV: return L.is_latent() ? (int64_t)c.a_heads * c.a_vdim * c.a_kv_rank : -1;
+        case MI355_HW_L_CNORM: return L.is_latent() ? c.a_kv_rank : -1;
         case MI355_HW_D_CONV: return L.has_delta() ? (int64_t)L.conv_channels() * c.d_conv : -1;
         case MI355_HW_D_A_LOG: return L.has_delta() ? c.d_heads : -1;
         case MI355_HW_D_DT_BIAS: return L.has_delta() ? (c.d_decay_channels ? c.d_heads * c.d_dim : c.d_heads) : -1;
@@ -208,6 +242,7 @@ int ensure_capacity(HModel* m, int T, int n_out) {
         HCHECK(grow(m->q, t * (size_t)m->max_q * m->esize()));
         HCHECK(grow(m->mix, t * (size_t)m->max_mix * m->esize()));
         HCHECK(grow(m->act, t * (size_t)m->max_ff * m->esize()));
+        HCHECK(grow(m->att, t * (size_t)m->max_att * m->esize()));
         HCHECK(grow(m->tok_seq, t * 4));
         m->cap_t = T;
     }
@@ -235,7 +270,17 @@ int32_t mi355_hybrid_in_proj_rows(const mi355_hybrid_layer* layer, int32_t* offs
 void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_layer* layers) {
     if (!cfg || !layers || cfg->width <= 0 || cfg->vocab <= 0 || cfg->n_layers <= 0 || cfg->block_size <= 0 || cfg->state_slots <= 0) return nullptr;
     if (cfg->dtype != MI355_DTYPE_F32 && cfg->dtype != MI355_DTYPE_BF16) return nullptr;
-    for (int i = 0; i < cfg->n_layers; ++i) if (!layer_ok(layers[i])) return nullptr;
+    for (int i = 0; i < cfg->n_layers; ++i) {
+        if (!layer_ok(layers[i])) return nullptr;
+        const int sw = layers[i].share_with;                   // the lender has weights of its own and the same shape
+        if (sw && (sw > cfg->n_layers || sw - 1 == i || layers[sw - 1].share_with)) return nullptr;
+        if (sw) {
+            mi355_hybrid_layer a = layers[i], b = layers[sw - 1];
+            a.share_with = b.share_with = 0;
+            if (std::memcmp(&a, &b, sizeof(a)) != 0) return nullptr;
+        }
+    }
+    if (cfg->residual_form < 0 || cfg->residual_form > 1 || cfg->norm_groups < 0 || (cfg->norm_groups > 1 && cfg->width % cfg->norm_groups)) return nullptr;
     HModel* m = new HModel();
     m->cfg = *cfg;
     m->layers.resize(cfg->n_layers);
@@ -246,12 +291,23 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
         const mi355_hybrid_layer& c = L.c;
         L.in_rows = in_proj_parts(c, L.off);
         L.out_k = 0;
-        if (L.has_attn()) L.out_k += c.a_heads * c.a_vdim;
+        if (L.uses_pages()) L.out_k += c.a_heads * c.a_vdim;
         if (L.has_delta()) L.out_k += c.d_heads * c.d_vdim;
         if (c.mixer == MI355_HYB_MIX_MINGRU) L.out_k = c.g_width;
         m->max_in_rows = std::max(m->max_in_rows, L.in_rows);
         m->max_mix = std::max(m->max_mix, L.out_k);
-        if (L.has_attn()) m->max_q = std::max(m->max_q, c.a_heads * c.a_dim);
+        if (L.has_attn() || L.is_conv_attn()) m->max_q = std::max(m->max_q, c.a_heads * c.a_dim);
+        if (L.is_latent()) {
+            m->max_q = std::max(m->max_q, c.a_heads * (c.a_kv_rank + c.a_rot_dim));
+            m->max_aux1 = std::max(m->max_aux1, c.a_heads * c.a_kv_rank);
+            m->max_att = std::max(m->max_att, c.a_heads * c.a_kv_rank);
+            m->max_o = std::max(m->max_o, c.a_heads * c.a_vdim);
+        }
+        if (L.is_conv_attn()) {
+            m->max_conv = std::max(m->max_conv, L.a_conv_channels());
+            m->max_o = std::max(m->max_o, c.a_heads * (c.a_talk ? c.a_kv_heads : 1) * c.a_vdim);
+            L.conv_off = off; off += (int64_t)L.a_conv_channels() * (c.a_conv - 1);
+        }
         if (L.has_delta()) {
             if (c.d_decay_channels) m->max_aux1 = std::max(m->max_aux1, c.d_heads * c.d_dim);
             if (c.d_gate == MI355_HYB_GATE_SIGMOID_LR) m->max_aux2 = std::max(m->max_aux2, c.d_heads * c.d_vdim);
@@ -278,7 +334,7 @@ void mi355_hybrid_destroy(void* mp) {
         for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.k_pages, L.v_pages}) if (p) (void)hipFree(p);
     }
     for (void* p : {m->embed.p, m->final_norm.p, m->head.p, (void*)m->state, (void*)m->prep, (void*)m->x, (void*)m->proj, (void*)m->aux1, (void*)m->aux2,
-                    (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, (void*)m->tok_seq})
+                    (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, m->att, (void*)m->tok_seq})
         if (p) (void)hipFree(p);
     delete m;
 }
@@ -306,7 +362,7 @@ int mi355_hybrid_set_rope_tables(void* mp, int32_t layer, const float* cos_t, co
     HModel* m = static_cast<HModel*>(mp);
     if (!m || layer < 0 || layer >= (int)m->layers.size() || !cos_t || !sin_t || n_positions <= 0) return -1;
     HLayer& L = m->layers[layer];
-    if (!L.has_attn() || L.c.a_rot_dims <= 0) return -2;
+    if (!L.rotates() || L.c.share_with) return -2;
     drop_graphs(m);
     const size_t bytes = (size_t)n_positions * (L.c.a_rot_dims / 2) * 4;
     HHIP(hipDeviceSynchronize());
@@ -326,7 +382,7 @@ int64_t mi355_hybrid_cache_bytes(void* mp, int32_t num_blocks) {
     if (!m || num_blocks < 0) return -1;
     int64_t b = m->slot_floats * 4 * m->cfg.state_slots;
     for (const HLayer& L : m->layers)
-        if (L.has_attn()) b += (int64_t)num_blocks * m->cfg.block_size * L.c.a_kv_heads * (L.c.a_dim + L.c.a_vdim) * (int64_t)m->esize();
+        if (L.uses_pages()) b += (int64_t)num_blocks * m->cfg.block_size * (L.k_row() + L.v_row()) * (int64_t)m->esize();
     return b;
 }
 
@@ -336,12 +392,14 @@ int mi355_hybrid_alloc_cache(void* mp, int32_t num_blocks) {
     HHIP(hipDeviceSynchronize());
     drop_graphs(m);
     for (HLayer& L : m->layers) {
-        if (!L.has_attn()) continue;
-        const size_t rows = (size_t)num_blocks * m->cfg.block_size * L.c.a_kv_heads;
-        HCHECK(grow(L.k_pages, rows * L.c.a_dim * m->esize()));
-        HCHECK(grow(L.v_pages, rows * L.c.a_vdim * m->esize()));
-        HHIP(hipMemset(L.k_pages, 0, rows * L.c.a_dim * m->esize()));
-        HHIP(hipMemset(L.v_pages, 0, rows * L.c.a_vdim * m->esize()));
+        if (!L.uses_pages()) continue;
+        const size_t rows = (size_t)num_blocks * m->cfg.block_size;
+        HCHECK(grow(L.k_pages, rows * L.k_row() * m->esize()));
+        HHIP(hipMemset(L.k_pages, 0, rows * L.k_row() * m->esize()));
+        if (L.v_row() > 0) {
+            HCHECK(grow(L.v_pages, rows * L.v_row() * m->esize()));
+            HHIP(hipMemset(L.v_pages, 0, rows * L.v_row() * m->esize()));
+        }
     }
     const size_t sb = (size_t)m->slot_floats * 4 * m->cfg.state_slots;
     HCHECK(grow(m->state, sb));
@@ -360,11 +418,14 @@ static int forward_check(HModel* m, const uint32_t* tokens, const int64_t* posit
     if (!m->state || !m->embed.p || !m->final_norm.p || !m->head.p) return -3;
     if ((int64_t)max_blocks * m->cfg.block_size < max_context_len) return -4;
     for (const HLayer& L : m->layers) {
-        const int need[] = {MI355_HW_NORM1, MI355_HW_IN_PROJ, MI355_HW_OUT_PROJ};
-        for (int s : need) if (!L.w[s].p) return -3;
-        for (int s = MI355_HW_NORM2; s < MI355_HW_COUNT; ++s)
-            if (s != MI355_HW_IN_BIAS && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
-        if (L.has_attn() && (!L.k_pages || (L.c.a_rot_dims > 0 && L.n_pos < max_context_len))) return -4;
+        const HLayer& WL = L.c.share_with ? m->layers[L.c.share_with - 1] : L;
+        if (!L.c.share_with) {
+            const int need[] = {MI355_HW_NORM1, MI355_HW_IN_PROJ, MI355_HW_OUT_PROJ};
+            for (int s : need) if (!L.w[s].p) return -3;
+            for (int s = MI355_HW_NORM2; s < MI355_HW_COUNT; ++s)
+                if (s != MI355_HW_IN_BIAS && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
+        }
+        if (L.uses_pages() && (!L.k_pages || (L.rotates() && WL.n_pos < max_context_len))) return -4;
     }
     return ensure_capacity(m, T, n_out);
 }
@@ -383,20 +444,63 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
     for (size_t li = 0; li < m->layers.size(); ++li) {
         HLayer& L = m->layers[li];
         const mi355_hybrid_layer& c = L.c;
-        auto f = [&](int which) { return static_cast<const float*>(L.w[which].p); };
+        const HLayer& WL = c.share_with ? m->layers[c.share_with - 1] : L;          // whose weights (and rope tables) the layer runs on
+        auto f = [&](int which) { return static_cast<const float*>(WL.w[which].p); };
         const int ldp = L.in_rows;
-        HCHECK(mi355_hyb_linear(m->proj, ldp, xin, xin_dt, W, L.w[MI355_HW_IN_PROJ].p, f(MI355_HW_IN_BIAS), T, L.in_rows, W, dt, stream));
+        HCHECK(mi355_hyb_linear(m->proj, ldp, xin, xin_dt, W, WL.w[MI355_HW_IN_PROJ].p, f(MI355_HW_IN_BIAS), T, L.in_rows, W, dt, stream));
         int mix_col = 0;
         if (L.has_attn()) {
             HCHECK(mi355_hyb_attn_prepare(m->q, L.k_pages, L.v_pages, m->proj, ldp, L.off[P_AQ], L.off[P_AK], L.off[P_AV],
                                           c.a_qk_norm ? f(MI355_HW_A_QNORM) : nullptr, c.a_qk_norm ? f(MI355_HW_A_KNORM) : nullptr,
-                                          L.cos_t, L.sin_t, positions, slot_mapping, T, c.a_heads, c.a_kv_heads, c.a_dim, c.a_vdim,
+                                          WL.cos_t, WL.sin_t, positions, slot_mapping, T, c.a_heads, c.a_kv_heads, c.a_dim, c.a_vdim,
                                           c.a_rot_dims, eps, dt, stream));
             HCHECK(mi355_hyb_window_attention(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens, cu_seqlens_q,
                                               m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, c.a_heads,
                                               c.a_kv_heads, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window, c.a_scale,
                                               c.mixer == MI355_HYB_MIX_PARALLEL ? c.a_out_scale : 1.f, dt, stream));
             mix_col = c.a_heads * c.a_vdim;
+        }
+        if (L.is_latent()) {
+            // absorbed form: q_abs[t, h] = W_uk,h^T q_h (one launch over the heads), attention over the latent rows themselves with
+            // ONE shared key/value head (keys [latent | rotated part], values = the latent part of the same page row), then W_uv,h
+            // on every head's latent-sized output, the head gate, and the output projection
+            const int R = c.a_kv_rank, dq = R + c.a_rot_dim, H = c.a_heads;
+            HCHECK(mi355_hyb_linear_batched(m->aux1, H * R, R, m->proj + L.off[P_AQ], MI355_DTYPE_F32, ldp, c.a_dim + c.a_rot_dim,
+                                            WL.w[MI355_HW_L_UKT].p, (int64_t)R * c.a_dim, T, R, c.a_dim, H, dt, stream));
+            HCHECK(mi355_hyb_latent_prepare(m->q, L.k_pages, m->proj, ldp, L.off[P_AQ], L.off[P_AK], m->aux1, f(MI355_HW_L_CNORM), WL.cos_t,
+                                            WL.sin_t, positions, slot_mapping, T, H, c.a_dim, c.a_rot_dim, R, c.a_rot_dims,
+                                            c.a_rot_interleaved, eps, dt, stream));
+            HCHECK(mi355_hyb_window_attention_ex(m->att, dt, H * R, 0, m->q, L.k_pages, L.k_pages, block_tables, context_lens, cu_seqlens_q,
+                                                 m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, H, 1, dq, R,
+                                                 m->cfg.block_size, max_blocks, c.a_window, c.a_scale, 1.f, dq, dq, c.a_softcap, 0, dt, stream));
+            HCHECK(mi355_hyb_linear_batched(m->o, H * c.a_vdim, c.a_vdim, m->att, dt, H * R, R, WL.w[MI355_HW_L_UV].p,
+                                            (int64_t)c.a_vdim * R, T, c.a_vdim, R, H, dt, stream));
+            if (c.a_head_gate) HCHECK(mi355_hyb_head_gate(m->mix, dt, m->o, m->proj + L.off[P_G], ldp, T, H, c.a_vdim, stream));
+            else HCHECK(mi355_hyb_head_gate(m->mix, dt, m->o, nullptr, 0, T, H, c.a_vdim, stream));
+        }
+        if (L.is_conv_attn()) {
+            const int C = L.a_conv_channels(), H = c.a_heads, G = c.a_kv_heads;
+            float* conv_state = m->state + L.conv_off;
+            HCHECK(mi355_hyb_conv(m->conv, m->proj, ldp, L.off[P_AQ], f(MI355_HW_A_CONV), conv_state, m->slot_floats, context_lens,
+                                  cu_seqlens_q, state_slots, m->tok_seq, num_seqs, T, C, c.a_conv, 0, stream));
+            HCHECK(mi355_hyb_conv_state_update(conv_state, m->slot_floats, m->proj, ldp, L.off[P_AQ], context_lens, cu_seqlens_q,
+                                               state_slots, num_seqs, C, c.a_conv, stream));
+            HCHECK(mi355_hyb_attn_prepare_whole(m->q, L.k_pages, L.v_pages, m->conv, C, 0, H * c.a_dim, (H + G) * c.a_dim,
+                                                c.a_qk_norm ? f(MI355_HW_A_QNORM) : nullptr, c.a_qk_norm ? f(MI355_HW_A_KNORM) : nullptr,
+                                                slot_mapping, T, H, G, c.a_dim, c.a_vdim, c.a_v_unit, eps, dt, stream));
+            if (c.a_talk) {
+                // mixed head weights: every head's weights against the values of every key/value head, then the mix of those outputs
+                HCHECK(mi355_hyb_window_attention_ex(m->o, MI355_DTYPE_F32, H * G * c.a_vdim, 0, m->q, L.k_pages, L.v_pages, block_tables,
+                                                     context_lens, cu_seqlens_q, m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr,
+                                                     num_seqs, T, H, G, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window,
+                                                     c.a_scale, 1.f, 0, 0, c.a_softcap, 1, dt, stream));
+                HCHECK(mi355_hyb_head_mix(m->mix, dt, m->o, f(MI355_HW_A_TALK), T, H, G, c.a_vdim, stream));
+            } else {
+                HCHECK(mi355_hyb_window_attention_ex(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens,
+                                                     cu_seqlens_q, m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, H,
+                                                     G, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window, c.a_scale, 1.f, 0, 0,
+                                                     c.a_softcap, 0, dt, stream));
+            }
         }
         if (L.has_delta()) {
             const int C = L.conv_channels();
@@ -408,14 +512,14 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             const float* decay_in = m->proj + L.off[P_A];
             int ldd = ldp;
             if (c.d_decay_channels) {
-                HCHECK(mi355_hyb_linear(m->aux1, c.d_heads * c.d_dim, m->proj + L.off[P_A], MI355_DTYPE_F32, ldp, L.w[MI355_HW_D_A2].p,
+                HCHECK(mi355_hyb_linear(m->aux1, c.d_heads * c.d_dim, m->proj + L.off[P_A], MI355_DTYPE_F32, ldp, WL.w[MI355_HW_D_A2].p,
                                         nullptr, T, c.d_heads * c.d_dim, c.d_a_rank, dt, stream));
                 decay_in = m->aux1; ldd = c.d_heads * c.d_dim;
             }
             const float* gate_in = m->proj + L.off[P_G];
             int ldg = ldp;
             if (c.d_gate == MI355_HYB_GATE_SIGMOID_LR) {
-                HCHECK(mi355_hyb_linear(m->aux2, c.d_heads * c.d_vdim, m->proj + L.off[P_G], MI355_DTYPE_F32, ldp, L.w[MI355_HW_D_G2].p,
+                HCHECK(mi355_hyb_linear(m->aux2, c.d_heads * c.d_vdim, m->proj + L.off[P_G], MI355_DTYPE_F32, ldp, WL.w[MI355_HW_D_G2].p,
                                         nullptr, T, c.d_heads * c.d_vdim, c.d_g_rank, dt, stream));
                 gate_in = m->aux2; ldg = c.d_heads * c.d_vdim;
             }
@@ -428,19 +532,26 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
         if (c.mixer == MI355_HYB_MIX_MINGRU)
             HCHECK(mi355_hyb_mingru(m->mix, dt, m->state + L.state_off, m->slot_floats, m->proj, ldp, L.off[0], L.off[1], L.off[2],
                                     context_lens, cu_seqlens_q, state_slots, num_seqs, T, c.g_width, stream));
-        HCHECK(mi355_hyb_linear(m->y, W, m->mix, dt, L.out_k, L.w[MI355_HW_OUT_PROJ].p, nullptr, T, W, L.out_k, dt, stream));
-        HCHECK(mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(MI355_HW_NORM1), T, W, eps, stream));
+        auto residual = [&](int norm_slot) -> int {
+            if (m->cfg.residual_form == 1)
+                return mi355_hyb_resid_norm(m->x, bf ? m->xcopy : nullptr, m->y, W, f(norm_slot), T, W, m->cfg.norm_groups, m->cfg.resid_alpha, eps, stream);
+            return mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(norm_slot), T, W, eps, stream);
+        };
+        HCHECK(mi355_hyb_linear(m->y, W, m->mix, dt, L.out_k, WL.w[MI355_HW_OUT_PROJ].p, nullptr, T, W, L.out_k, dt, stream));
+        HCHECK(residual(MI355_HW_NORM1));
         if (c.mlp_kind) {
-            HCHECK(mi355_hyb_linear(m->gu, 2 * c.mlp_ff, xin, xin_dt, W, L.w[MI355_HW_MLP_GATE_UP].p, nullptr, T, 2 * c.mlp_ff, W, dt, stream));
-            HCHECK(mi355_hyb_clamped_glu(m->act, dt, m->gu, T, c.mlp_ff, c.mlp_limit, c.mlp_alpha, stream));
-            HCHECK(mi355_hyb_linear(m->y, W, m->act, dt, c.mlp_ff, L.w[MI355_HW_MLP_DOWN].p, nullptr, T, W, c.mlp_ff, dt, stream));
-            HCHECK(mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(MI355_HW_NORM2), T, W, eps, stream));
+            HCHECK(mi355_hyb_linear(m->gu, 2 * c.mlp_ff, xin, xin_dt, W, WL.w[MI355_HW_MLP_GATE_UP].p, nullptr, T, 2 * c.mlp_ff, W, dt, stream));
+            if (c.mlp_kind == 2) HCHECK(mi355_hyb_gelu_glu(m->act, dt, m->gu, T, c.mlp_ff, stream));
+            else HCHECK(mi355_hyb_clamped_glu(m->act, dt, m->gu, T, c.mlp_ff, c.mlp_limit, c.mlp_alpha, stream));
+            HCHECK(mi355_hyb_linear(m->y, W, m->act, dt, c.mlp_ff, WL.w[MI355_HW_MLP_DOWN].p, nullptr, T, W, c.mlp_ff, dt, stream));
+            HCHECK(residual(MI355_HW_NORM2));
         }
         if (layer_trace)
             HHIP(hipMemcpyAsync(layer_trace + li * (size_t)T * W, m->x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, reinterpret_cast<hipStream_t>(stream)));
     }
     if (n_out > 0) {
-        HCHECK(mi355_hyb_gather_norm(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W, eps, stream));
+        HCHECK(mi355_hyb_gather_group_norm(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W,
+                                           m->cfg.norm_groups, eps, stream));
         HCHECK(mi355_hyb_linear(logits, m->cfg.vocab, m->xn, dt, W, m->head.p, nullptr, n_out, m->cfg.vocab, W, dt, stream));
     }
     return 0;

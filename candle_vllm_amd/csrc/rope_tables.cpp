@@ -3,6 +3,7 @@
 // reference's arithmetic -- inverse frequencies rounded to f32, angle = f32(position) * f32(inv_freq), cos / sin of
 // that f32 angle -- so the tables agree with a candle build to the last bit of libm.  The tables are f32
 // [n_positions, rotary_dim / 2]; the kernels (fused QKV epilogue, mi355_rope_inplace) only ever read them.
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <vector>
@@ -144,16 +145,30 @@ extern "C" int mi355_rope_tables(float* cos_out, float* sin_out, int32_t rotary_
 
 // ABI guard: struct sizes as this build of the header sees them (hand-written mirrors compare against it)
 // The same tables with frequencies, angles and their cosines / sines taken in f64 and rounded once: for host layers whose angles are
-// not tied to the reference's f32 arithmetic (include/mi355_hybrid.h).  Default, linear and llama3 scaling.
+// not tied to the reference's f32 arithmetic (include/mi355_hybrid.h).  Default, linear, llama3 and yarn scaling (yarn: the
+// frequency blend between the indices where a wavelength makes beta_fast / beta_slow turns over the original length, and the
+// amplitude 0.1 ln(factor) + 1 (times attn_factor) on both tables).
 extern "C" int mi355_rope_tables_f64(float* cos_out, float* sin_out, int32_t rotary_dim, int32_t n_positions, double rope_theta,
                                      const mi355_rope_scaling* sc, int32_t max_seq_len, int32_t max_position_embeddings) {
     if (!cos_out || !sin_out || rotary_dim <= 0 || (rotary_dim & 1) || n_positions <= 0 || rope_theta <= 0) return 1;
     const int type = sc ? sc->type : MI355_ROPE_DEFAULT;
-    if (type != MI355_ROPE_DEFAULT && type != MI355_ROPE_LINEAR && type != MI355_ROPE_LLAMA3) return 1;
+    if (type != MI355_ROPE_DEFAULT && type != MI355_ROPE_LINEAR && type != MI355_ROPE_LLAMA3 && type != MI355_ROPE_YARN) return 1;
     const int half = rotary_dim / 2;
     std::vector<double> f(half);
     for (int i = 0; i < half; ++i) f[i] = pow(rope_theta, -2.0 * (double)i / (double)rotary_dim);
-    double pos_div = 1.0;
+    double pos_div = 1.0, amplitude = 1.0;
+    if (type == MI355_ROPE_YARN) {
+        if (sc->factor <= 0) return 1;
+        const double orig = original_max(sc, max_position_embeddings, max_seq_len);
+        const double fast = sc->beta_fast > 0 ? sc->beta_fast : 32.0, slow = sc->beta_slow > 0 ? sc->beta_slow : 1.0;
+        auto turn_index = [&](double turns) { return (double)rotary_dim * log(orig / (2.0 * M_PI * turns)) / (2.0 * log(rope_theta)); };
+        const double lo = std::max(floor(turn_index(fast)), 0.0), hi = std::min(ceil(turn_index(slow)), (double)rotary_dim - 1.0);
+        for (int i = 0; i < half; ++i) {
+            const double ramp = std::min(std::max(((double)i - lo) / std::max(hi - lo, 0.001), 0.0), 1.0);
+            f[i] = f[i] / sc->factor * ramp + f[i] * (1.0 - ramp);
+        }
+        amplitude = (sc->factor <= 1.0 ? 1.0 : 0.1 * log(sc->factor) + 1.0) * (sc->attn_factor > 0 ? sc->attn_factor : 1.0);
+    }
     if (type == MI355_ROPE_LINEAR) { if (sc->factor <= 0) return 1; pos_div = sc->factor; }
     if (type == MI355_ROPE_LLAMA3) {
         if (sc->factor <= 0 || sc->low_freq_factor <= 0 || sc->high_freq_factor <= 0) return 1;
@@ -171,8 +186,8 @@ extern "C" int mi355_rope_tables_f64(float* cos_out, float* sin_out, int32_t rot
     for (int p = 0; p < n_positions; ++p)
         for (int i = 0; i < half; ++i) {
             const double th = (double)p / pos_div * f[i];
-            cos_out[(size_t)p * half + i] = (float)cos(th);
-            sin_out[(size_t)p * half + i] = (float)sin(th);
+            cos_out[(size_t)p * half + i] = (float)(cos(th) * amplitude);
+            sin_out[(size_t)p * half + i] = (float)(sin(th) * amplitude);
         }
     return 0;
 }

@@ -1,7 +1,8 @@
 """Python harness over the `mi355_hybrid_*` handle (include/mi355_hybrid.h): layer-list models whose layers mix tokens by
-sliding-window attention with a sink, a gated delta rule, a minGRU, or attention and delta rule side by side.  The Sogodra design
-is read here: its config.json (`architecture`, `layers`, `norm`, `vocab`, `width`) becomes the C structs, its tensors are
-concatenated into the host layer's slots.  No CPU fallback; torch only holds device buffers."""
+sliding-window attention with a sink, a gated delta rule, a minGRU, attention and delta rule side by side, latent attention, or
+attention behind a short convolution with mixed head weights.  The Sogodra and Vivazen designs are read here: a design's
+config.json (`architecture`, `layers`, `norm`, `vocab`, `width`, ...) becomes the C structs, its tensors are concatenated into the
+host layer's slots.  No CPU fallback; torch only holds device buffers."""
 import ctypes
 import json
 import os
@@ -13,11 +14,13 @@ import torch
 from ._lib import lib, HybridConfig, HybridLayer, RopeScaling
 
 DT_F32, DT_BF16 = 0, 2
-MIX_PARALLEL, MIX_MINGRU, MIX_DELTA, MIX_ATTENTION = 0, 1, 2, 3
+MIX_PARALLEL, MIX_MINGRU, MIX_DELTA, MIX_ATTENTION, MIX_LATENT, MIX_CONV_ATTENTION = 0, 1, 2, 3, 4, 5
 GATE_SILU, GATE_SIGMOID_LR = 0, 1
-ROPE_DEFAULT, ROPE_LLAMA3 = 0, 2
+ROPE_DEFAULT, ROPE_LLAMA3, ROPE_YARN = 0, 2, 4
 (HW_EMBED, HW_FINAL_NORM, HW_HEAD, HW_NORM1, HW_NORM2, HW_IN_PROJ, HW_IN_BIAS, HW_OUT_PROJ, HW_A_QNORM, HW_A_KNORM, HW_A_SINK, HW_D_CONV,
- HW_D_A_LOG, HW_D_DT_BIAS, HW_D_NORM, HW_D_A2, HW_D_G2, HW_MLP_GATE_UP, HW_MLP_DOWN) = range(19)
+ HW_D_A_LOG, HW_D_DT_BIAS, HW_D_NORM, HW_D_A2, HW_D_G2, HW_MLP_GATE_UP, HW_MLP_DOWN, HW_A_CONV, HW_A_TALK, HW_L_UKT, HW_L_UV,
+ HW_L_CNORM) = range(24)
+MLP_CLAMPED_GLU, MLP_GELU_GLU = 1, 2
 
 # constants the Sogodra design fixes
 SOGODRA_GLU_ALPHA = 1.702          # y = g sigmoid(1.702 g) (u + 1)
@@ -68,8 +71,32 @@ def _bf16_bits(a):
     return ((u + 0x7FFF + ((u >> 16) & 1)) >> 16).astype(np.uint16)
 
 
+class HeadTranspose:
+    """a slot entry: tensor `name` [heads * a, b] stored as [heads, b, a] (every head's block transposed)"""
+
+    def __init__(self, name, heads):
+        self.name, self.heads = name, int(heads)
+
+    def bits(self, bits, shapes):
+        rows, cols = shapes[self.name]
+        a = np.asarray(bits[self.name], np.uint16).reshape(self.heads, rows // self.heads, cols)
+        return np.ascontiguousarray(a.transpose(0, 2, 1)).reshape(-1)
+
+
 class SogodraSpec:
     """config.json of a Sogodra model -> layer structs + the tensor names behind every weight slot"""
+    residual_form, resid_alpha, norm_groups = 0, 1.0, 1          # x <- x + norm(sub(x)), one RMS over the whole vector
+
+    @staticmethod
+    def rope_scaling(rot):
+        rs = RopeScaling()
+        sc = rot.get("scaling")
+        if sc:
+            rs.type, rs.factor, rs.low_freq_factor, rs.high_freq_factor = ROPE_LLAMA3, float(sc["factor"]), float(sc["low"]), float(sc["high"])
+            rs.original_max_position_embeddings = float(sc["original"])
+        else:
+            rs.type = ROPE_DEFAULT
+        return rs
 
     def __init__(self, cfg, shapes):
         """cfg: the parsed config.json; shapes: tensor name -> shape (which optional tensors exist, ranks of low-rank parts)"""
@@ -145,6 +172,92 @@ class SogodraSpec:
         return L, slots, rope
 
 
+class VivazenSpec:
+    """config.json of a Vivazen model -> layer structs + the tensor names behind every weight slot.  The design: the norm sits behind
+    the residual sum, x <- N(alpha x + sub(x)), N = RMS norm over `norm.groups` parts of the vector; layers are latent attention
+    (window, sink, head gate, interleaved rotation with yarn scaling on the rotated part) or attention behind a convolution (norms
+    over the whole q / k projections, unit values, capped scores, mixed head weights); gelu-tanh gate/up feed-forward; a layer with
+    `weights_of` runs on that layer's tensors with a cache of its own."""
+    residual_form = 1
+
+    @staticmethod
+    def rope_scaling(rot):
+        rs = RopeScaling()
+        sc = rot.get("scaling")
+        if sc:
+            rs.type, rs.factor, rs.original_max_position_embeddings = ROPE_YARN, float(sc["factor"]), float(sc["original"])
+            rs.beta_fast, rs.beta_slow, rs.attn_factor = float(sc["fast"]), float(sc["slow"]), 1.0
+        else:
+            rs.type = ROPE_DEFAULT
+        return rs
+
+    def __init__(self, cfg, shapes):
+        if cfg.get("architecture") != "Vivazen":
+            raise ValueError("not a Vivazen config")
+        self.cfg = cfg
+        self.width, self.vocab = int(cfg["width"]), int(cfg["vocab"])
+        self.eps, self.norm_groups = float(cfg["norm"]["eps"]), int(cfg["norm"].get("groups", 1))
+        self.resid_alpha = float(cfg.get("postln_alpha", 1.0))
+        self.layers, self.slots, self.rope = [], [], []
+        entries = cfg["layers"]
+        for i, lc in enumerate(entries):
+            src = i
+            while "weights_of" in entries[src]:                 # the layer whose tensors this one runs on
+                src = int(entries[src]["weights_of"])
+                if src == i:
+                    raise ValueError(f"layer {i}: weights_of runs in a circle")
+            L, slots, rope = self._layer("l%d." % src, lc, shapes)
+            if src != i:
+                L.share_with, slots, rope = src + 1, {}, None
+            self.layers.append(L)
+            self.slots.append(slots)
+            self.rope.append(rope)
+
+    def _layer(self, p, lc, shapes):
+        L, slots, rope = HybridLayer(), {HW_NORM1: [p + "norm1"]}, None
+        c, kind, q = lc["mixer"], lc["type"], p + "mix."
+        L.a_heads, L.a_dim, L.a_vdim, L.a_scale, L.a_out_scale = int(c["heads"]), int(c["dim"]), int(c["vdim"]), float(c["scale"]), 1.0
+        L.a_window = int(c["mask"]["size"]) if c.get("mask") else 0
+        L.a_softcap = float(c.get("softcap") or 0.0)
+        L.a_has_sink = int(q + "sink" in shapes)
+        if L.a_has_sink:
+            slots[HW_A_SINK] = [q + "sink"]
+        if kind == "latent_attention":
+            L.mixer = MIX_LATENT
+            L.a_kv_heads, L.a_kv_rank, L.a_rot_dim = 1, int(c["kv_rank"]), int(c["rot_dim"])
+            rope = c.get("rot")
+            L.a_rot_dims, L.a_rot_interleaved = (int(rope["dims"]) if rope else 0), 1
+            L.a_head_gate = int(q + "g" in shapes)
+            slots[HW_IN_PROJ] = [q + "q", q + "dkv"] + ([q + "g"] if L.a_head_gate else [])
+            slots[HW_L_UKT], slots[HW_L_UV], slots[HW_L_CNORM] = [HeadTranspose(q + "uk", L.a_heads)], [q + "uv"], [q + "dkv.norm"]
+        elif kind == "attention":
+            L.mixer = MIX_CONV_ATTENTION
+            L.a_kv_heads, L.a_conv = int(c["kv_heads"]), int(c.get("conv") or 1)
+            L.a_qk_norm = L.a_norm_whole = int(q + "q.norm" in shapes)
+            L.a_v_unit, L.a_talk = 1, int(q + "talk" in shapes)
+            slots[HW_IN_PROJ] = [q + "q", q + "k", q + "v"]
+            if L.a_qk_norm:
+                slots[HW_A_QNORM], slots[HW_A_KNORM] = [q + "q.norm"], [q + "k.norm"]
+            if L.a_conv > 1 or q + "q.conv" in shapes:
+                slots[HW_A_CONV] = [q + "q.conv", q + "k.conv", q + "v.conv"]
+            if L.a_talk:
+                slots[HW_A_TALK] = [q + "talk"]
+        else:
+            raise ValueError(f"layer type {kind!r} is not part of the design")
+        slots[HW_OUT_PROJ] = [q + "o"]
+        mlp = lc.get("mlp")
+        if mlp:
+            if mlp.get("kind") != "dense":
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not part of the design")
+            L.mlp_kind, L.mlp_ff = MLP_GELU_GLU, int(mlp["ff"])
+            slots[HW_NORM2] = [p + "norm2"]
+            slots[HW_MLP_GATE_UP], slots[HW_MLP_DOWN] = [p + "mlp.gate", p + "mlp.up"], [p + "mlp.down"]
+        return L, slots, rope
+
+
+SPECS = {"Sogodra": SogodraSpec, "Vivazen": VivazenSpec}       # config.json `architecture` -> its reader
+
+
 class HybridModel:
     stateful = True                       # its layers carry state from token to token: a sequence needs a state slot
 
@@ -155,7 +268,8 @@ class HybridModel:
         n = len(spec.layers)
         self._layers = (HybridLayer * n)(*spec.layers)
         c = HybridConfig(width=spec.width, vocab=spec.vocab, n_layers=n, dtype=self.dtype, block_size=self.block_size,
-                         state_slots=self.state_slots, norm_eps=spec.eps, unit_eps=SOGODRA_UNIT_EPS)
+                         state_slots=self.state_slots, norm_eps=spec.eps, unit_eps=SOGODRA_UNIT_EPS,
+                         residual_form=int(spec.residual_form), resid_alpha=float(spec.resid_alpha), norm_groups=int(spec.norm_groups))
         self.h = lib.mi355_hybrid_create(ctypes.byref(c), self._layers)
         if not self.h:
             raise RuntimeError("mi355_hybrid_create refused the configuration")
@@ -172,7 +286,9 @@ class HybridModel:
     def from_pretrained(cls, model_dir, dtype="bfloat16", block_size=DEFAULT_BLOCK_SIZE, state_slots=4):
         cfg = json.load(open(os.path.join(model_dir, "config.json")))
         tensors = read_safetensors(os.path.join(model_dir, "model.safetensors"))
-        spec = SogodraSpec(cfg, {k: v[1] for k, v in tensors.items()})
+        if cfg.get("architecture") not in SPECS:
+            raise ValueError(f"architecture {cfg.get('architecture')!r} is not a layer-list design (known: {sorted(SPECS)})")
+        spec = SPECS[cfg["architecture"]](cfg, {k: v[1] for k, v in tensors.items()})
         m = cls(spec, dtype=dtype, block_size=block_size, state_slots=state_slots)
         m.load_tensors({k: v[0] for k, v in tensors.items()}, {k: v[1] for k, v in tensors.items()})
         return m
@@ -206,7 +322,8 @@ class HybridModel:
                     mats = [np.asarray(bits[nm], np.uint16).reshape(shapes[nm]) for nm in names]
                     self._put(i, which, np.concatenate(mats, axis=0))
                 else:
-                    self._put(i, which, np.concatenate([np.asarray(bits[nm], np.uint16).reshape(-1) for nm in names]))
+                    self._put(i, which, np.concatenate([nm.bits(bits, shapes) if isinstance(nm, HeadTranspose)
+                                                        else np.asarray(bits[nm], np.uint16).reshape(-1) for nm in names]))
 
     def load_state_dict_f32(self, W):
         """W: tensor name -> f32 ndarray (tests, synthetic weights); rounded to bf16"""
@@ -214,8 +331,8 @@ class HybridModel:
 
     # ---- cache
     def ensure_rope(self, n_positions):
-        """cos / sin tables of every attention layer up to n_positions (the framework's table builder in its f64 form; llama3 scaling when
-        the config has `rot.scaling`)"""
+        """cos / sin tables of every rotating layer up to n_positions (the framework's table builder in its f64 form; the scaling of
+        the design when the config has `rot.scaling`)"""
         if n_positions <= self.rope_positions:
             return
         n = max(int(n_positions), 2 * self.rope_positions, 256)
@@ -224,13 +341,7 @@ class HybridModel:
                 continue
             half = L.a_rot_dims // 2
             cos, sin = np.zeros((n, half), np.float32), np.zeros((n, half), np.float32)
-            sc = rot.get("scaling")
-            rs = RopeScaling()
-            if sc:
-                rs.type, rs.factor, rs.low_freq_factor, rs.high_freq_factor = ROPE_LLAMA3, float(sc["factor"]), float(sc["low"]), float(sc["high"])
-                rs.original_max_position_embeddings = float(sc["original"])
-            else:
-                rs.type = ROPE_DEFAULT
+            rs = self.spec.rope_scaling(rot)
             _check(lib.mi355_rope_tables_f64(cos.ctypes.data, sin.ctypes.data, L.a_rot_dims, n, float(rot["base"]), ctypes.byref(rs), n, n),
                    "rope_tables")
             _check(lib.mi355_hybrid_set_rope_tables(self.h, i, cos.ctypes.data, sin.ctypes.data, n), "set_rope_tables")

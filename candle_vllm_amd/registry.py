@@ -5,11 +5,22 @@ import json
 import os
 
 _REGISTRY = {}
+_COMPONENT = {}
 
 
-def register(name, loader):
-    """loader(model_dir, config, **options) -> model"""
+def register(name, loader, component=None):
+    """loader(model_dir, config, **options) -> model; component: the part of the library that serves the model when it can be built
+    alone (`__graft_entry__.COMPONENTS`), None = the whole library"""
     _REGISTRY[name] = loader
+    _COMPONENT[name] = component
+
+
+def component_of(config):
+    """which part of the library a config needs (None: the whole library, or nothing registered)"""
+    for name in architectures_of(config):
+        if name in _REGISTRY:
+            return _COMPONENT[name]
+    return None
 
 
 def architectures_of(config):
@@ -33,7 +44,7 @@ def load_model(model_dir, **options):
                      f"registered: {registered()}")
 
 
-def _load_sogodra(model_dir, config, dtype="bfloat16", block_size=None, state_slots=4, **_):
+def _load_layer_list(model_dir, config, dtype="bfloat16", block_size=None, state_slots=4, **_):
     from .hybrid_model import HybridModel, DEFAULT_BLOCK_SIZE
     return HybridModel.from_pretrained(model_dir, dtype=dtype, block_size=block_size or DEFAULT_BLOCK_SIZE, state_slots=state_slots)
 
@@ -43,6 +54,7 @@ def _load_dense_llama(model_dir, config, dtype="bfloat16", **options):
     return load_dense_llama(model_dir, config, dtype=dtype, **options)
 
 
-register("Sogodra", _load_sogodra)
+for _name in ("Sogodra", "Vivazen"):
+    register(_name, _load_layer_list, component="hybrid")
 for _name in ("LlamaForCausalLM", "MistralForCausalLM", "Qwen2ForCausalLM"):
     register(_name, _load_dense_llama)

@@ -1,6 +1,8 @@
 /* C ABI of the layer-list ("hybrid") host layer: decoder-only models whose config lists, layer by layer, which token mixer a
  * layer has -- sliding-window attention with a softmax sink, a gated delta rule (recurrent matrix state), a minGRU (recurrent vector
- * state), or attention and delta rule side by side -- and which feed-forward.  The Sogodra design is the first user.
+ * state), attention and delta rule side by side, latent attention (keys and values read off one cached latent vector per token), or
+ * attention behind a short convolution whose heads' softmax weights are mixed -- and which feed-forward.  The Sogodra and Vivazen
+ * designs are its users.
  *
  * What differs from the llama-family host layers (mi355_llama_*, mi355_dense_*):
  *   - the residual stream, norms, attention scores, decays, gates of a recurrence and the recurrent state are f32 in both dtypes;
@@ -23,6 +25,12 @@ extern "C" {
 #define MI355_HYB_MIX_MINGRU 1
 #define MI355_HYB_MIX_DELTA 2
 #define MI355_HYB_MIX_ATTENTION 3  /* the attention branch alone */
+#define MI355_HYB_MIX_LATENT 4     /* latent attention: the pages hold [latent c (a_kv_rank) | rotated key part (a_rot_dim)] per token;
+                                      head h's key is W_uk,h c and its value W_uv,h c.  Computed in the absorbed form: the query
+                                      carries W_uk,h^T q_h, the attention runs over the latent rows themselves (one shared key/value
+                                      head of a_kv_rank + a_rot_dim / a_kv_rank dimensions), W_uv,h is applied to its output */
+#define MI355_HYB_MIX_CONV_ATTENTION 5 /* q, k, v pass a short causal convolution (a_conv taps, no activation), then attention with
+                                      the a_* switches below; the convolution's last inputs live in the state slot */
 
 #define MI355_HYB_GATE_SILU 0      /* output gate silu(W_g h), full rank                */
 #define MI355_HYB_GATE_SIGMOID_LR 1 /* output gate sigmoid(W_g2 (W_g1 h)), low rank     */
@@ -46,9 +54,23 @@ typedef struct mi355_hybrid_layer {
     float d_out_scale;
     /* minGRU */
     int32_t g_width;
-    /* feed-forward: 0 = none, 1 = dense clamped gate/up with y = g sigmoid(act_alpha g) (u + 1)                   */
+    /* feed-forward: 0 = none, 1 = dense clamped gate/up with y = g sigmoid(act_alpha g) (u + 1),
+                     2 = dense gate/up with y = gelu_tanh(g) u                                                     */
     int32_t mlp_kind, mlp_ff;
     float mlp_limit, mlp_alpha;
+    /* more switches of the attention branch (all 0 = the plain form) */
+    int32_t a_rot_interleaved;     /* rotated pairs are (2i, 2i + 1) instead of (i, i + a_rot_dims / 2)                   */
+    int32_t a_kv_rank, a_rot_dim;  /* latent attention: latent size; rotated dimensions per query head = the shared key part
+                                      (a_dim = the unrotated dimensions per head, a_rot_dims <= a_rot_dim of them turn)    */
+    int32_t a_head_gate;           /* head h's output times sigmoid((W_g x)_h), W_g [heads, width] in the input projection */
+    int32_t a_conv;                /* taps of the convolution behind q, k, v                                               */
+    int32_t a_norm_whole;          /* a_qk_norm is ONE RMS norm over all of q (and of k), weights [heads * dim]            */
+    int32_t a_v_unit;              /* every value head is divided by its root mean square before it is cached             */
+    float a_softcap;               /* > 0: score <- cap tanh(score / cap)                                                  */
+    int32_t a_talk;                /* weight_h <- sum_g talk[h, g] weight_g after the softmax; head h applies its mixed
+                                      weights to the values of its own key/value head                                      */
+    int32_t share_with;            /* 0: the layer has weights; n > 0: it runs on layer n - 1's weights (and rope tables) with
+                                      pages and state of its own                                                           */
 } mi355_hybrid_layer;
 
 typedef struct mi355_hybrid_config {
@@ -58,6 +80,10 @@ typedef struct mi355_hybrid_config {
     int32_t state_slots;           /* recurrent-state slots (live sequences)                                       */
     float norm_eps;
     float unit_eps;                /* eps inside the root of the unit norm of q and k in the delta rule            */
+    int32_t residual_form;         /* 0: x <- x + norm(sub(x));  1: x <- norm(resid_alpha x + sub(x))                */
+    float resid_alpha;
+    int32_t norm_groups;           /* the layer norms and the last norm take the RMS over this many equal consecutive parts
+                                      of the vector separately (0 or 1: over the whole vector)                       */
 } mi355_hybrid_config;
 
 /* weight slots: `layer` = -1 for the three global ones */
@@ -81,12 +107,19 @@ typedef struct mi355_hybrid_config {
 #define MI355_HW_D_G2 16           /* [heads * vdim, g_rank]                                                        */
 #define MI355_HW_MLP_GATE_UP 17    /* [2 ff, width]: gate rows, then up rows                                        */
 #define MI355_HW_MLP_DOWN 18       /* [width, ff]                                                                   */
-#define MI355_HW_COUNT 19
+#define MI355_HW_A_CONV 19         /* [q channels + k channels + v channels, taps], last column = the current token */
+#define MI355_HW_A_TALK 20         /* [heads, heads]                                                                */
+#define MI355_HW_L_UKT 21          /* [heads, kv_rank, dim]: per head the TRANSPOSE of its block of W_uk [heads dim, kv_rank] */
+#define MI355_HW_L_UV 22           /* [heads vdim, kv_rank]                                                         */
+#define MI355_HW_L_CNORM 23        /* [kv_rank] weight of the latent's RMS norm                                      */
+#define MI355_HW_COUNT 24
 
 void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_layer* layers);
 void mi355_hybrid_destroy(void* model);
 /* rows of a layer's concatenated input projection, and where each part starts: parts = attention q, k, v, delta q, k, v, beta,
- * decay (a or a1), gate (g or g1) for the attention / delta / parallel mixers; z, x, g for the minGRU.  offsets[9], -1 = absent */
+ * decay (a or a1), gate (g or g1) for the attention / delta / parallel mixers; z, x, g for the minGRU; q (heads x (dim + rot_dim)),
+ * the latent down-projection (kv_rank + rot_dim) in the k part and the head gate in the gate part for latent attention.
+ * offsets[9], -1 = absent */
 int32_t mi355_hybrid_in_proj_rows(const mi355_hybrid_layer* layer, int32_t* offsets);
 /* HOST bf16 bits (a checkpoint tensor), n elements; converted to the storage type of the slot */
 int mi355_hybrid_set_weight(void* model, int32_t layer, int32_t which, const uint16_t* host_bf16, int64_t n);
@@ -148,6 +181,57 @@ int mi355_hyb_window_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
                                const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, int32_t num_seqs, int32_t num_tokens,
                                int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size, int32_t max_blocks,
                                int32_t window, float scale, float out_scale, int32_t dtype, int64_t stream);
+/* the same with the remaining switches: k_ld / v_ld = elements per page row of the key / value pages (0: kv_heads x dim | vdim;
+ * latent attention passes the same pages for both with v_ld = k_ld), softcap (0 = none), cross_values: 1 = every query head's
+ * weights are applied to the values of EVERY key/value head c, out [T, heads, kv_heads, vdim] (what mi355_hyb_head_mix reads) */
+int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                                  const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                                  const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, int32_t num_seqs,
+                                  int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
+                                  int32_t max_blocks, int32_t window, float scale, float out_scale, int32_t k_ld, int32_t v_ld,
+                                  float softcap, int32_t cross_values, int32_t dtype, int64_t stream);
+/* out (dt_out) [T, heads x vdim] = sum_g talk[h, g] a[t, g, kv head of h, :],  a f32 [T, heads, kv_heads, vdim]: mixing the heads'
+ * softmax weights before the value product is the same as mixing, per key/value head, the outputs the unmixed weights give */
+int mi355_hyb_head_mix(void* out, int32_t out_dtype, const float* a, const float* talk, int32_t num_tokens, int32_t heads,
+                       int32_t kv_heads, int32_t vdim, int64_t stream);
+/* out (dt_out) [T, heads x vdim] = in f32 [T, heads x vdim] times sigmoid(gate_in[t, h]) per head (gate_in NULL: a plain copy) */
+int mi355_hyb_head_gate(void* out, int32_t out_dtype, const float* in, const float* gate_in, int32_t ldg, int32_t num_tokens,
+                        int32_t heads, int32_t vdim, int64_t stream);
+/* attention behind a convolution: src f32 [T, ld] holds q | k | v rows (offsets q_off, k_off, v_off).  q and k: RMS norm over the WHOLE
+ * row part (heads x dim, kv_heads x dim) with weights of that size (NULL = no norm); v: every head divided by its root mean square when
+ * v_unit.  q -> q_out (dt) [T, heads, dim], k, v -> the pages at slot_mapping.  No rotation */
+int mi355_hyb_attn_prepare_whole(void* q_out, void* k_pages, void* v_pages, const float* src, int32_t ld, int32_t q_off, int32_t k_off,
+                                 int32_t v_off, const float* q_norm_w, const float* k_norm_w, const int64_t* slot_mapping,
+                                 int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t v_unit, float eps,
+                                 int32_t dtype, int64_t stream);
+/* latent attention: proj f32 [T, ldp] holds per head [dim unrotated | rot_dim rotated] query rows at q_off and the down-projection
+ * [kv_rank | rot_dim] at c_off; q_abs f32 [T, heads, kv_rank] = the unrotated query parts already multiplied by W_uk^T.
+ * pages (dt) [.., kv_rank + rot_dim] at slot_mapping <- [RMS norm of the latent times c_norm_w | rotated key part];
+ * q_out (dt) [T, heads, kv_rank + rot_dim] <- [q_abs | rotated query part].  The first rot_dims of the rot_dim dimensions turn
+ * (pairs (2i, 2i+1) when interleaved), cos_t / sin_t [positions, rot_dims / 2] carry any amplitude */
+int mi355_hyb_latent_prepare(void* q_out, void* pages, const float* proj, int32_t ldp, int32_t q_off, int32_t c_off, const float* q_abs,
+                             const float* c_norm_w, const float* cos_t, const float* sin_t, const int64_t* positions,
+                             const int64_t* slot_mapping, int32_t num_tokens, int32_t heads, int32_t dim, int32_t rot_dim,
+                             int32_t kv_rank, int32_t rot_dims, int32_t interleaved, float eps, int32_t dtype, int64_t stream);
+/* `batch` independent products of one shape in one launch: out + z o_bs [T, ldo] = (a + z a_bs) [T, lda] . (w + z w_bs) [n, k]^T,
+ * strides in elements (per-head matrices: z = head) */
+int mi355_hyb_linear_batched(float* out, int32_t ldo, int64_t o_bs, const void* a, int32_t a_dtype, int32_t lda, int64_t a_bs,
+                             const void* w, int64_t w_bs, int32_t num_tokens, int32_t n, int32_t k, int32_t batch, int32_t dtype,
+                             int64_t stream);
+/* x f32 [T, width] <- group norm(alpha x + y) times w (the norm BEHIND the residual sum; `groups` equal consecutive parts, each with
+ * its own root mean square); xcopy: NULL or bf16 [T, width] */
+int mi355_hyb_resid_norm(float* x, void* xcopy, const float* y, int32_t ldy, const float* w, int32_t num_tokens, int32_t width,
+                         int32_t groups, float alpha, float eps, int64_t stream);
+/* mi355_hyb_gather_norm with the RMS taken over `groups` parts */
+int mi355_hyb_gather_group_norm(void* out, int32_t out_dtype, const float* x, const int32_t* rows, const float* w, int32_t n_rows,
+                                int32_t width, int32_t groups, float eps, int64_t stream);
+/* out (dt_out) [T, ff] = gelu_tanh(gu[:, j]) gu[:, ff + j] */
+int mi355_hyb_gelu_glu(void* out, int32_t out_dtype, const float* gu, int32_t num_tokens, int32_t ff, int64_t stream);
+/* mi355_hyb_conv_silu with the activation as an argument: 0 = none, 1 = silu */
+int mi355_hyb_conv(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* conv_state,
+                   int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                   const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t channels, int32_t taps, int32_t act,
+                   int64_t stream);
 /* 0: prompt-sized steps over bf16 pages take the generic kernel instead of the matrix-core one (A/B switch, process-wide; default 1) */
 void mi355_hyb_set_attention_mfma(int32_t on);
 /* short causal convolution over time per channel, then silu: out f32 [T, channels] from proj columns [off, off + channels);

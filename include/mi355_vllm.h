@@ -452,7 +452,7 @@ typedef struct mi355_rope_scaling {
 int32_t mi355_rope_table_len(const mi355_rope_scaling* sc, int32_t max_seq_len, int32_t max_position_embeddings);
 int mi355_rope_tables(float* cos_out_host, float* sin_out_host, int32_t rotary_dim, int32_t n_positions, double rope_theta,
                       const mi355_rope_scaling* sc /* NULL = default */, int32_t max_seq_len, int32_t max_position_embeddings);
-/* the same tables with frequencies and angles in f64, rounded once (default, linear and llama3 scaling; 1 for the others) */
+/* the same tables with frequencies and angles in f64, rounded once (default, linear, llama3 and yarn scaling; 1 for the others) */
 int mi355_rope_tables_f64(float* cos_out_host, float* sin_out_host, int32_t rotary_dim, int32_t n_positions, double rope_theta,
                           const mi355_rope_scaling* sc, int32_t max_seq_len, int32_t max_position_embeddings);
 /* `Config::effective_max_seq_len` (src/openai/models/mod.rs:663-702): max(base, round(original * factor)) for yarn with
