@@ -1,5 +1,5 @@
-"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, random weights) at layer
-sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
+"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, or Vivazen with
+`--hybrid-design vivazen`; random weights) at layer sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
 width, depth, head geometry, feed-forward size and vocabulary.  One GPU, bf16, synthetic data.  The default workload of bench.py and
 its one-line contract are not touched: this option prints its own JSON line.
 
@@ -17,6 +17,55 @@ SIZES = {
     "3b": dict(width=3072, heads=24, kv=8, dim=128, ff=8192, vocab=32000, window=2048, dheads=24, ddim=128, dvdim=128, gru=6144, layers="pgdp"),
     "8b": dict(width=4096, heads=32, kv=8, dim=128, ff=14336, vocab=32000, window=4096, dheads=32, ddim=128, dvdim=128, gru=8192, layers="pgdp"),
 }
+
+
+# Vivazen at the same widths: latent attention (heads x (dim + rot) queries over [kv_rank | rot] page rows, window) and attention behind
+# a convolution (heads / kv heads as above, capped scores, mixed head weights), gelu gate/up; the fourth layer runs on the first one's weights
+VIVAZEN = {
+    "1b": dict(l_heads=16, l_dim=64, l_rot=64, l_rank=192, l_vdim=64, taps=4, layers="laal"),
+    "3b": dict(l_heads=24, l_dim=64, l_rot=64, l_rank=192, l_vdim=64, taps=4, layers="laal"),
+    "8b": dict(l_heads=32, l_dim=128, l_rot=64, l_rank=192, l_vdim=128, taps=4, layers="laal"),
+}
+
+
+def vivazen_config(s, v):
+    lat = {"dim": v["l_dim"], "heads": v["l_heads"], "kv_rank": v["l_rank"], "rot_dim": v["l_rot"], "vdim": v["l_vdim"],
+           "scale": (v["l_dim"] + v["l_rot"]) ** -0.5, "mask": {"size": s["window"]},
+           "rot": {"base": 50000.0, "dims": v["l_rot"], "scaling": {"factor": 4.0, "fast": 32.0, "original": 2048, "slow": 1.0}}}
+    att = {"conv": v["taps"], "dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv"], "scale": s["dim"] ** -0.5, "softcap": 50.0, "vdim": s["dim"]}
+    mlp = {"ff": s["ff"], "kind": "dense"}
+    layers, first = [], {}
+    for i, c in enumerate(v["layers"]):
+        e = {"type": "latent_attention" if c == "l" else "attention", "mixer": lat if c == "l" else att, "mlp": mlp}
+        if c == "l" and "l" in first:
+            e["weights_of"] = first["l"]
+        first.setdefault(c, i)
+        layers.append(e)
+    return {"architecture": "Vivazen", "layers": layers, "norm": {"eps": 1e-5, "groups": 4}, "postln_alpha": 3.0, "vocab": s["vocab"], "width": s["width"]}
+
+
+def vivazen_shapes(cfg):
+    W, sh = cfg["width"], {}
+    sh["embed"], sh["final.norm"], sh["head"] = (cfg["vocab"], W), (W,), (cfg["vocab"], W)
+    for i, lc in enumerate(cfg["layers"]):
+        if "weights_of" in lc:
+            continue
+        p, c = "l%d." % i, lc["mixer"]
+        q = p + "mix."
+        sh[p + "norm1"] = (W,)
+        if lc["type"] == "latent_attention":
+            H, d, r, vd, rank = c["heads"], c["dim"], c["rot_dim"], c["vdim"], c["kv_rank"]
+            sh[q + "q"], sh[q + "dkv"], sh[q + "dkv.norm"], sh[q + "uk"], sh[q + "uv"] = (H * (d + r), W), (rank + r, W), (rank,), (H * d, rank), (H * vd, rank)
+            sh[q + "sink"], sh[q + "g"], sh[q + "o"] = (H,), (H, W), (W, H * vd)
+        else:
+            H, G, d, vd, t = c["heads"], c["kv_heads"], c["dim"], c["vdim"], c["conv"]
+            for n, rows in (("q", H * d), ("k", G * d), ("v", G * vd)):
+                sh[q + n], sh[q + n + ".conv"] = (rows, W), (rows, t)
+            sh[q + "q.norm"], sh[q + "k.norm"], sh[q + "talk"], sh[q + "o"] = (H * d,), (G * d,), (H, H), (W, H * vd)
+        if lc.get("mlp"):
+            ff = lc["mlp"]["ff"]
+            sh[p + "norm2"], sh[p + "mlp.gate"], sh[p + "mlp.up"], sh[p + "mlp.down"] = (W,), (ff, W), (ff, W), (W, ff)
+    return sh
 
 
 def sogodra_config(s):
@@ -69,8 +118,8 @@ def build_hybrid(cfg, max_tokens, slots):
     """random weights generated on the GPU, concatenated as the loader does it, handed over as device bf16"""
     import torch
     from candle_vllm_amd import hybrid_model as hm
-    shapes = sogodra_shapes(cfg)
-    spec = hm.SogodraSpec(cfg, shapes)
+    shapes = vivazen_shapes(cfg) if cfg["architecture"] == "Vivazen" else sogodra_shapes(cfg)
+    spec = hm.SPECS[cfg["architecture"]](cfg, shapes)
     m = hm.HybridModel(spec, dtype="bfloat16", block_size=64, state_slots=slots)
     g = torch.Generator(device="cuda").manual_seed(7)
     nbytes = 0
@@ -81,11 +130,14 @@ def build_hybrid(cfg, max_tokens, slots):
             return (1 + 0.02 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
         if name == "embed":
             return torch.randn(shape, generator=g, device="cuda").to(torch.bfloat16)
+        if name.endswith(".talk"):
+            return (torch.eye(shape[0], device="cuda") + 0.1 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
         s = 0.5 if name.endswith(".conv") else (fan ** -0.5 if len(shape) > 1 else 0.3)
         return (s * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
 
     def put(layer, which, names, axis=0):
         nonlocal nbytes
+        names = [n.name if isinstance(n, hm.HeadTranspose) else n for n in names]       # random values: the transposed layout is as random
         ts = [rnd(shapes[n], n) if n else None for n in names]
         if which == hm.HW_IN_BIAS:
             rows = [shapes[p][0] for p in spec.slots[layer][hm.HW_IN_PROJ]]
@@ -113,16 +165,17 @@ def time_calls(call, sync, reps=5, settle_ms=200.0):
     return sorted(d)[len(d) // 2]
 
 
-def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16):
+def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16, design="sogodra"):
     import torch
     from candle_vllm_amd import dense_model as DM
     from candle_vllm_amd.block_engine import BlockEngine
     from candle_vllm_amd.step_engine import StepEngine
     from oracle.dense_llama import DenseConfig
     s = SIZES[name]
-    cfg = sogodra_config(s)
+    cfg = vivazen_config(s, VIVAZEN[name]) if design == "vivazen" else sogodra_config(s)
     rng = np.random.default_rng(5)
-    out = {"size": name, "shape": s, "prompt_tokens": T, "decode_batch": B, "decode_ctx": ctx}
+    out = {"size": name, "design": design, "shape": dict(s, **(VIVAZEN[name] if design == "vivazen" else {})), "prompt_tokens": T, "decode_batch": B,
+           "decode_ctx": ctx}
     sync = torch.cuda.synchronize
     # ---- hybrid: prompt step, then B sequences decoding behind ctx tokens
     hyb, wbytes = build_hybrid(cfg, max(T, B * (ctx + 1024)) + 64, slots=max(4, B))
@@ -153,7 +206,7 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16):
     del eng, hyb
     torch.cuda.empty_cache()
     # ---- the llama host layer at equal size
-    n_layers = len(s["layers"])
+    n_layers = len(cfg["layers"])
     dc = DenseConfig(hidden=s["width"], n_layers=n_layers, n_heads=s["heads"], n_kv_heads=s["kv"], head_dim=s["dim"], intermediate=s["ff"],
                      vocab=s["vocab"], max_seq=8192, block_size=64)
     nblk = B * (-(-(ctx + 64) // 64)) + (-(-T // 64)) + 2
@@ -189,7 +242,10 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16):
     return out
 
 
-def main(sizes="1b,3b", prompt_tokens=2048, batch=8, ctx=2048):
-    res = [run_size(n.strip(), T=prompt_tokens, B=batch, ctx=ctx) for n in sizes.split(",") if n.strip()]
+def main(sizes="1b,3b", prompt_tokens=2048, batch=8, ctx=2048, design="sogodra"):
+    if design not in ("sogodra", "vivazen"):
+        raise SystemExit("--hybrid-design: sogodra or vivazen")
+    res = [run_size(n.strip(), T=prompt_tokens, B=batch, ctx=ctx, design=design) for n in sizes.split(",") if n.strip()]
     print(json.dumps({"metric": "hybrid_vs_llama_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
-                      "note": "Sogodra layer-list host layer beside the 16-bit llama host layer at equal sizes; eager steps", "sizes": res}))
+                      "note": "%s layer-list host layer beside the 16-bit llama host layer at equal sizes; the hybrid side's decode steps replay "
+                              "a hipGraph, the rest runs eagerly" % design.capitalize(), "sizes": res}))

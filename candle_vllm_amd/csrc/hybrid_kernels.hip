@@ -335,6 +335,22 @@ __global__ __launch_bounds__(256) void resid_norm_kernel(float* x, uint16_t* xco
     const int t = blockIdx.x, part = width / groups;
     float* xr = x + (size_t)t * width;
     const float* yr = y + (size_t)t * ldy;
+    if (groups >= (int)(blockDim.x >> 6)) {                    // a wave per part, parts in turn: no workgroup-wide exchange at all
+        const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+        for (int g = wave; g < groups; g += nw) {
+            float ss = 0.f;
+            for (int i = lane; i < part; i += 64) { const float v = fmaf(alpha, xr[g * part + i], yr[g * part + i]); ss = fmaf(v, v, ss); }
+            ss = wave_sum(ss);
+            const float inv = 1.f / sqrtf(ss / (float)part + eps);
+            for (int i = lane; i < part; i += 64) {
+                const int c = g * part + i;
+                const float v = fmaf(alpha, xr[c], yr[c]) * inv * w[c];
+                xr[c] = v;
+                if (xcopy) xcopy[(size_t)t * width + c] = f32_to_bf16(v);
+            }
+        }
+        return;
+    }
     for (int g0 = 0; g0 < groups; g0 += 64) {
         const int gn = min(64, groups - g0);
         for (int g = 0; g < gn; ++g) {
@@ -476,7 +492,8 @@ template <> struct Vec16<float> {
 // value.  VEC (head sizes that are multiples of 16 bytes): rows are read 16 bytes at a time; for the value sum the wave's lanes
 // are (key, 16-byte chunk of the row) pairs -- 64 / cp2 keys per pass -- and the keys' partial sums are added by lane exchanges.
 // DQ > 0 (VEC, d = DQ): the query sits in registers, so a key's score costs its 16-byte loads and d FMAs and nothing else.
-template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
+// NV > 1 (cross mode): the head's weights are applied to the values of NV key/value heads; the scores are computed once.
+template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
     constexpr int EPV = Vec16<TC>::N;
     constexpr int NACC = VEC ? EPV : 8;
     extern __shared__ __align__(16) float smem[];
@@ -490,7 +507,7 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
     const int pos = (int)p.ctx[s] - n_new + (t - (int)p.cu_q[s]);
     const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
     const int g = h / (p.H / p.G);
-    const int gv = p.cross ? (int)blockIdx.z : g, oh = p.cross ? h * p.G + gv : h;
+    const int gv0 = p.cross ? (int)blockIdx.z * NV : g, oh0 = p.cross ? h * p.G + gv0 : h;
     const TC* q = static_cast<const TC*>(p.q) + ((size_t)t * p.H + h) * p.d;
     for (int i = threadIdx.x; i < p.d; i += blockDim.x) qs[i] = ld<TC>(q, i);
     __syncthreads();
@@ -502,9 +519,11 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
     const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
     const int cp2 = p.cp2, chunk = lane & (cp2 - 1), ksub = lane / cp2, kpp = 64 / cp2;     // VEC only
     const bool chunk_ok = chunk * EPV < p.vd;
-    float m = -INFINITY, l = 0.f, acc[NACC];
+    float m = -INFINITY, l = 0.f, acc[NV][NACC];
 #pragma unroll
-    for (int e = 0; e < NACC; ++e) acc[e] = 0.f;
+    for (int n = 0; n < NV; ++n)
+#pragma unroll
+        for (int e = 0; e < NACC; ++e) acc[n][e] = 0.f;
     for (int j0 = lo + wave * 64; j0 <= pos; j0 += NW * 64) {
         const int j = j0 + lane;
         float sc = -INFINITY;
@@ -538,7 +557,9 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
         const float corr = (m == -INFINITY) ? 0.f : expf(m - mn);
         l = l * corr + wave_sum(pj);
 #pragma unroll
-        for (int e = 0; e < NACC; ++e) acc[e] *= corr;
+        for (int n = 0; n < NV; ++n)
+#pragma unroll
+            for (int e = 0; e < NACC; ++e) acc[n][e] *= corr;
         m = mn;
         const int cnt = min(64, pos - j0 + 1);
         if (VEC) {
@@ -547,19 +568,25 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
                 const float pv = __shfl(pj, jj & 63);
                 const size_t pr = (size_t)__shfl(page_row, jj & 63);
                 if (jj < cnt && chunk_ok) {
-                    float x[EPV];
-                    Vec16<TC>::load(static_cast<const TC*>(p.v_pages) + pr * p.v_ld + gv * p.vd + chunk * EPV, x);
 #pragma unroll
-                    for (int e = 0; e < EPV; ++e) acc[e] = fmaf(pv, x[e], acc[e]);
+                    for (int n = 0; n < NV; ++n) {
+                        float x[EPV];
+                        Vec16<TC>::load(static_cast<const TC*>(p.v_pages) + pr * p.v_ld + (gv0 + n) * p.vd + chunk * EPV, x);
+#pragma unroll
+                        for (int e = 0; e < EPV; ++e) acc[n][e] = fmaf(pv, x[e], acc[n][e]);
+                    }
                 }
             }
         } else {
             for (int jj = 0; jj < cnt; ++jj) {
                 const float pv = __shfl(pj, jj);
                 const size_t pr = (size_t)__shfl(page_row, jj);
-                const TC* vr = static_cast<const TC*>(p.v_pages) + pr * p.v_ld + gv * p.vd;
 #pragma unroll
-                for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) acc[e] = fmaf(pv, ld<TC>(vr, c), acc[e]); }
+                for (int n = 0; n < NV; ++n) {
+                    const TC* vr = static_cast<const TC*>(p.v_pages) + pr * p.v_ld + (gv0 + n) * p.vd;
+#pragma unroll
+                    for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) acc[n][e] = fmaf(pv, ld<TC>(vr, c), acc[n][e]); }
+                }
             }
         }
     }
@@ -567,13 +594,19 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
     if (VEC) {
         for (int off = cp2; off < 64; off <<= 1)
 #pragma unroll
-            for (int e = 0; e < NACC; ++e) acc[e] += __shfl_xor(acc[e], off);
+            for (int n = 0; n < NV; ++n)
+#pragma unroll
+                for (int e = 0; e < NACC; ++e) acc[n][e] += __shfl_xor(acc[n][e], off);
         if (ksub == 0 && chunk_ok)
 #pragma unroll
-            for (int e = 0; e < EPV; ++e) pacc[wave * p.vd + chunk * EPV + e] = acc[e];
+            for (int n = 0; n < NV; ++n)
+#pragma unroll
+                for (int e = 0; e < EPV; ++e) pacc[(wave * NV + n) * p.vd + chunk * EPV + e] = acc[n][e];
     } else {
 #pragma unroll
-        for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) pacc[wave * p.vd + c] = acc[e]; }
+        for (int n = 0; n < NV; ++n)
+#pragma unroll
+            for (int e = 0; e < NACC; ++e) { const int c = lane + 64 * e; if (c < p.vd) pacc[(wave * NV + n) * p.vd + c] = acc[n][e]; }
     }
     __syncthreads();
     if (wave == 0) {
@@ -582,12 +615,14 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
         float L = p.sink ? expf(p.sink[h] - M) : 0.f;
         float cw[NW];
         for (int w = 0; w < NW; ++w) { cw[w] = pm[w] == -INFINITY ? 0.f : expf(pm[w] - M); L += pl[w] * cw[w]; }
-        const size_t base = (size_t)t * p.ldo + p.out_off + (size_t)oh * p.vd;
-        for (int col = lane; col < p.vd; col += 64) {
-            float o = 0.f;
-            for (int w = 0; w < NW; ++w) o += pacc[w * p.vd + col] * cw[w];
-            if (p.out_f32) st<float>(static_cast<float*>(p.out), base + col, o / L * p.out_scale);
-            else st<uint16_t>(static_cast<uint16_t*>(p.out), base + col, o / L * p.out_scale);
+        for (int n = 0; n < NV; ++n) {
+            const size_t base = (size_t)t * p.ldo + p.out_off + (size_t)(oh0 + n) * p.vd;
+            for (int col = lane; col < p.vd; col += 64) {
+                float o = 0.f;
+                for (int w = 0; w < NW; ++w) o += pacc[(w * NV + n) * p.vd + col] * cw[w];
+                if (p.out_f32) st<float>(static_cast<float*>(p.out), base + col, o / L * p.out_scale);
+                else st<uint16_t>(static_cast<uint16_t*>(p.out), base + col, o / L * p.out_scale);
+            }
         }
     }
 }
@@ -599,7 +634,9 @@ template <typename TC, int NW, bool VEC, int DQ> __global__ __launch_bounds__(64
 //   P V: the probabilities go through LDS into A-fragment order as TWO bf16 planes (p = hi + lo, so the weights keep about 16 bits
 //   of mantissa), the 64 value rows are transposed through LDS ([column][key]) so that a B fragment is one 16-byte read.
 // The sink is applied at the end: denominator += exp(sink - max).
-template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention_mfma_kernel(AttnArgs p) {
+// NV > 1 (cross mode): the block applies its head's weights to the values of NV key/value heads one after the other -- Q K^T, the
+// softmax and the probability planes are made once per chunk, the transposed value tile in LDS is refilled per value head.
+template <int DK, int VT, int NV> __global__ __launch_bounds__(64) void window_attention_mfma_kernel(AttnArgs p) {
     constexpr int RS = 72;                                           // bf16 per LDS row: 64 keys + 8 of padding (144 bytes)
     __shared__ __align__(16) uint16_t Ph[16 * RS], Pl[16 * RS], Vt[VT * 16 * RS];
     const int lane = threadIdx.x, m16 = lane & 15, kg = lane >> 4;
@@ -614,7 +651,7 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
     const int t0 = (int)p.cu_q[s] + b * 16, nq = min(16, (int)p.cu_q[s + 1] - t0);
     const int pos0 = (int)p.ctx[s] - n_new + b * 16;
     const int h = blockIdx.y, g = h / (p.H / p.G), d = p.d, vd = p.vd;
-    const int gv = p.cross ? (int)blockIdx.z : g, oh = p.cross ? h * p.G + gv : h;
+    const int gv0 = p.cross ? (int)blockIdx.z * NV : g, oh0 = p.cross ? h * p.G + gv0 : h;
     const uint16_t* Q = static_cast<const uint16_t*>(p.q);
     const uint16_t* K = static_cast<const uint16_t*>(p.k_pages);
     const uint16_t* V = static_cast<const uint16_t*>(p.v_pages);
@@ -624,14 +661,44 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
     for (int ks = 0; ks < DK; ++ks)
         qf[ks] = m16 < nq ? *reinterpret_cast<const uint4*>(Q + ((size_t)(t0 + m16) * p.H + h) * d + ks * 32 + 8 * kg) : uint4{0, 0, 0, 0};
     float mrow[4], lrow[4];
-    f32x4_t acc[VT];
+    f32x4_t acc[NV][VT];
 #pragma unroll
     for (int v = 0; v < 4; ++v) { mrow[v] = -INFINITY; lrow[v] = 0.f; }
 #pragma unroll
-    for (int c = 0; c < VT; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int n = 0; n < NV; ++n)
+#pragma unroll
+        for (int c = 0; c < VT; ++c) acc[n][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const int hi = pos0 + nq - 1;
     const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
     for (int j0 = lo; j0 <= hi; j0 += 64) {
+        // the 64 value rows of this chunk, transposed into LDS (zeros past the end: a stale NaN times a zero weight would poison the sum)
+        // (a value head's rows are requested into registers one head ahead of their use: the next head's loads are in flight while the
+        // current head multiplies)
+        uint4 vreg[VT * 2];
+        const int vkey = j0 + lane;
+        const bool vkv = vkey <= hi;
+        const uint16_t* vrow = V + (vkv ? (size_t)bt[vkey / p.bs] * p.bs + (vkey % p.bs) : 0) * p.v_ld + gv0 * vd;
+        auto fetch_values = [&](int n) {
+#pragma unroll
+            for (int c8 = 0; c8 < VT * 2; ++c8) vreg[c8] = vkv ? *reinterpret_cast<const uint4*>(vrow + n * vd + c8 * 8) : uint4{0, 0, 0, 0};
+        };
+        // transposing store: a word holds two neighbouring columns of this lane's key; the lane pair (2a, 2a + 1) swaps words, the
+        // even lane keeps the even column of both keys and the odd lane the odd column, so every lane writes ONE 4-byte word (two
+        // keys of one column) instead of two 2-byte halves
+        auto stage_values = [&]() {
+            const int col_odd = lane & 1, key_even = lane & ~1;
+#pragma unroll
+            for (int c8 = 0; c8 < VT * 2; ++c8) {
+                const uint32_t w[4] = {vreg[c8].x, vreg[c8].y, vreg[c8].z, vreg[c8].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w[e], 0xB1, 0xF, 0xF, true);   // quad_perm [1, 0, 3, 2]
+                    const uint32_t pair = col_odd ? ((other >> 16) | (w[e] & 0xFFFF0000u)) : ((w[e] & 0xFFFFu) | (other << 16));
+                    *reinterpret_cast<uint32_t*>(&Vt[(c8 * 8 + 2 * e + col_odd) * RS + key_even]) = pair;
+                }
+            }
+        };
+        fetch_values(0);
         f32x4_t sacc[4];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
@@ -646,23 +713,8 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
                 sacc[kt] = mfma_bf16(qf[ks], kf, sacc[kt]);
             }
         }
-        // the 64 value rows of this chunk, transposed into LDS (zeros past the end: a stale NaN times a zero weight would poison the sum)
-        {
-            const int key = j0 + lane;
-            const bool kv = key <= hi;
-            const size_t pr = kv ? (size_t)bt[key / p.bs] * p.bs + (key % p.bs) : 0;
-            const uint16_t* vr = V + pr * p.v_ld + gv * vd;
-#pragma unroll
-            for (int c8 = 0; c8 < VT * 2; ++c8) {
-                const uint4 x = kv ? *reinterpret_cast<const uint4*>(vr + c8 * 8) : uint4{0, 0, 0, 0};
-                const uint32_t w[4] = {x.x, x.y, x.z, x.w};
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    Vt[(c8 * 8 + 2 * e) * RS + lane] = (uint16_t)(w[e] & 0xFFFFu);
-                    Vt[(c8 * 8 + 2 * e + 1) * RS + lane] = (uint16_t)(w[e] >> 16);
-                }
-            }
-        }
+        stage_values();
+        if (NV > 1) fetch_values(1);
         // mask, scale, online softmax (rows 4 kg + v; this lane's keys: kt * 16 + m16)
         float mx[4], sc[4][4];
 #pragma unroll
@@ -697,21 +749,34 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
             lrow[v] = lrow[v] * corr + rs;
             mrow[v] = mn;
 #pragma unroll
-            for (int c = 0; c < VT; ++c) acc[c][v] *= corr;
+            for (int n = 0; n < NV; ++n)
+#pragma unroll
+                for (int c = 0; c < VT; ++c) acc[n][c][v] *= corr;
         }
         __syncthreads();
+        uint4 ah[2], al[2];
 #pragma unroll
         for (int k2 = 0; k2 < 2; ++k2) {
-            const uint4 ah = *reinterpret_cast<const uint4*>(&Ph[m16 * RS + k2 * 32 + 8 * kg]);
-            const uint4 al = *reinterpret_cast<const uint4*>(&Pl[m16 * RS + k2 * 32 + 8 * kg]);
-#pragma unroll
-            for (int c = 0; c < VT; ++c) {
-                const uint4 vf = *reinterpret_cast<const uint4*>(&Vt[(c * 16 + m16) * RS + k2 * 32 + 8 * kg]);
-                acc[c] = mfma_bf16(ah, vf, acc[c]);
-                acc[c] = mfma_bf16(al, vf, acc[c]);
-            }
+            ah[k2] = *reinterpret_cast<const uint4*>(&Ph[m16 * RS + k2 * 32 + 8 * kg]);
+            al[k2] = *reinterpret_cast<const uint4*>(&Pl[m16 * RS + k2 * 32 + 8 * kg]);
         }
-        __syncthreads();
+#pragma unroll
+        for (int n = 0; n < NV; ++n) {
+            if (n > 0) {
+                stage_values();
+                __syncthreads();
+                if (n + 1 < NV) fetch_values(n + 1);
+            }
+#pragma unroll
+            for (int k2 = 0; k2 < 2; ++k2)
+#pragma unroll
+                for (int c = 0; c < VT; ++c) {
+                    const uint4 vf = *reinterpret_cast<const uint4*>(&Vt[(c * 16 + m16) * RS + k2 * 32 + 8 * kg]);
+                    acc[n][c] = mfma_bf16(ah[k2], vf, acc[n][c]);
+                    acc[n][c] = mfma_bf16(al[k2], vf, acc[n][c]);
+                }
+            __syncthreads();
+        }
     }
     const float sink = p.sink ? p.sink[h] : -INFINITY;
 #pragma unroll
@@ -722,12 +787,15 @@ template <int DK, int VT> __global__ __launch_bounds__(64) void window_attention
         const float cm = expf(mrow[v] - M);
         const float L = lrow[v] * cm + (p.sink ? expf(sink - M) : 0.f);
         const float f = cm / L * p.out_scale;
-        const size_t base = (size_t)(t0 + r) * p.ldo + p.out_off + (size_t)oh * vd;
 #pragma unroll
-        for (int c = 0; c < VT; ++c) {
-            const float o = acc[c][v] * f;
-            if (p.out_f32) static_cast<float*>(p.out)[base + c * 16 + m16] = o;
-            else static_cast<uint16_t*>(p.out)[base + c * 16 + m16] = f32_to_bf16(o);
+        for (int n = 0; n < NV; ++n) {
+            const size_t base = (size_t)(t0 + r) * p.ldo + p.out_off + (size_t)(oh0 + n) * vd;
+#pragma unroll
+            for (int c = 0; c < VT; ++c) {
+                const float o = acc[n][c][v] * f;
+                if (p.out_f32) static_cast<float*>(p.out)[base + c * 16 + m16] = o;
+                else static_cast<uint16_t*>(p.out)[base + c * 16 + m16] = f32_to_bf16(o);
+            }
         }
     }
 }
@@ -1302,7 +1370,6 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
     AttnArgs p{out, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq, sink,
                num_seqs, heads, kv_heads, dim, vdim, block_size, max_blocks, window, scale, out_scale, 64, out_dtype == MI355_DTYPE_F32,
                k_ld, v_ld, softcap, cross};
-    const dim3 grid(T, heads, nz);
     hipStream_t s_ = to_stream(stream);
     const int epv = f ? 4 : 8;
     const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 &&
@@ -1312,30 +1379,51 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
     // prompt-sized steps over bf16 pages: the matrix-core kernel (a tile of 16 tokens never spans two sequences)
     if (!f && T >= 64 && dim % 32 == 0 && dim <= 256 && vdim % 16 == 0 && vdim <= 256 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
         (uintptr_t)v_pages % 16 == 0 && k_ld % 8 == 0 && v_ld % 8 == 0 && g_attn_mfma) {
-        const dim3 mgrid((T + 15) / 16 + num_seqs, heads, nz);
         const int dk = dim / 32, vt = vdim / 16;
-#define WM(DK, VT) window_attention_mfma_kernel<DK, VT><<<mgrid, 64, 0, s_>>>(p)
-#define WMV(DK) do { if (vt <= 2) { if (vt == 1) WM(DK, 1); else WM(DK, 2); } else if (vt <= 4) { if (vt == 3) WM(DK, 3); else WM(DK, 4); } \
-                     else if (vt <= 8) { if (vt <= 6) { if (vt == 5) WM(DK, 5); else WM(DK, 6); } else { if (vt == 7) WM(DK, 7); else WM(DK, 8); } } \
-                     else ok_shape = false; } while (0)
+        // cross mode: 4 or 2 value heads per block where the head sizes have such a build (dim <= 128, vdim <= 128), the rest of
+        // the key/value heads along z
+        const int nv = (cross && dk <= 4 && vt <= 8) ? (kv_heads % 4 == 0 ? 4 : kv_heads % 2 == 0 ? 2 : 1) : 1;
+        const dim3 mgrid((T + 15) / 16 + num_seqs, heads, nz / nv);
+#define WM1(DK, VT) window_attention_mfma_kernel<DK, VT, 1><<<mgrid, 64, 0, s_>>>(p)
+#define WMN(DK, VT) do { if (nv == 4) window_attention_mfma_kernel<DK, VT, 4><<<mgrid, 64, 0, s_>>>(p); \
+                         else if (nv == 2) window_attention_mfma_kernel<DK, VT, 2><<<mgrid, 64, 0, s_>>>(p); else WM1(DK, VT); } while (0)
+#define WMV(DK, WM) do { switch (vt) { case 1: WM(DK, 1); break; case 2: WM(DK, 2); break; case 3: WM(DK, 3); break; case 4: WM(DK, 4); break; \
+                                        case 5: WM(DK, 5); break; case 6: WM(DK, 6); break; case 7: WM(DK, 7); break; case 8: WM(DK, 8); break; \
+                                        default: ok_shape = false; } } while (0)
+        // value rows wider than 128 (latent attention: the latent itself is the value row): 16-column steps up to 256
+#define WMW(DK) do { switch (vt) { case 10: WM1(DK, 10); break; case 12: WM1(DK, 12); break; case 14: WM1(DK, 14); break; case 16: WM1(DK, 16); break; \
+                                   default: ok_shape = false; } } while (0)
         bool ok_shape = true;
-        switch (dk) { case 1: WMV(1); break; case 2: WMV(2); break; case 3: WMV(3); break; case 4: WMV(4); break; case 6: WMV(6); break;
-                      case 8: WMV(8); break; default: ok_shape = false; }
+        if (vt > 8) {
+            switch (dk) { case 4: WMW(4); break; case 5: WMW(5); break; case 6: WMW(6); break; case 7: WMW(7); break; case 8: WMW(8); break;
+                          default: ok_shape = false; }
+        } else {
+            switch (dk) { case 1: WMV(1, WMN); break; case 2: WMV(2, WMN); break; case 3: WMV(3, WMN); break; case 4: WMV(4, WMN); break;
+                          case 6: WMV(6, WM1); break; case 8: WMV(8, WM1); break; default: ok_shape = false; }
+        }
+#undef WMW
 #undef WMV
-#undef WM
+#undef WMN
+#undef WM1
         if (ok_shape) { LAUNCH_OK(); return 0; }
     }
     // few (token, head) pairs (decoding batches): eight waves share a window instead of four
     const bool wide = (int64_t)T * heads < 2048;
     const int dq = !vec ? 0 : dim == 64 ? 64 : dim == 128 ? 128 : 0;
-#define WA3(TC, NW, VEC, DQ) window_attention_kernel<TC, NW, VEC, DQ><<<grid, 64 * NW, (size_t)(((dim + 3) & ~3) + 2 * NW + NW * vdim) * sizeof(float), s_>>>(p)
-#define WA2(TC, NW) do { if (!vec) WA3(TC, NW, false, 0); else if (dq == 64) WA3(TC, NW, true, 64); else if (dq == 128) WA3(TC, NW, true, 128); \
+    // cross mode with 16-byte rows: 4 or 2 value heads per workgroup, the rest of the key/value heads along z
+    int nv = (cross && vec) ? (kv_heads % 4 == 0 ? 4 : kv_heads % 2 == 0 ? 2 : 1) : 1;
+    if ((size_t)8 * nv * vdim * sizeof(float) > 32768) nv = 1;          // the waves' partial sums must fit the workgroup's LDS
+    const dim3 ggrid(T, heads, nz / nv);
+#define WA4(TC, NW, VEC, DQ, NV) window_attention_kernel<TC, NW, VEC, DQ, NV><<<ggrid, 64 * NW, (size_t)(((dim + 3) & ~3) + 2 * NW + NW * NV * vdim) * sizeof(float), s_>>>(p)
+#define WA3(TC, NW, VEC, DQ) do { if (nv == 4) WA4(TC, NW, VEC, DQ, 4); else if (nv == 2) WA4(TC, NW, VEC, DQ, 2); else WA4(TC, NW, VEC, DQ, 1); } while (0)
+#define WA2(TC, NW) do { if (!vec) WA4(TC, NW, false, 0, 1); else if (dq == 64) WA3(TC, NW, true, 64); else if (dq == 128) WA3(TC, NW, true, 128); \
                          else WA3(TC, NW, true, 0); } while (0)
 #define WA(TC) do { if (wide) WA2(TC, 8); else WA2(TC, 4); } while (0)
     if (f) WA(float); else WA(uint16_t);
 #undef WA
 #undef WA2
 #undef WA3
+#undef WA4
     LAUNCH_OK(); return 0;
 }
 
