@@ -31,8 +31,8 @@ VIVAZEN = {
 def vivazen_config(s, v):
     lat = {"dim": v["l_dim"], "heads": v["l_heads"], "kv_rank": v["l_rank"], "rot_dim": v["l_rot"], "vdim": v["l_vdim"],
            "scale": (v["l_dim"] + v["l_rot"]) ** -0.5, "mask": {"size": s["window"]},
-           "rot": {"base": 50000.0, "dims": v["l_rot"], "scaling": {"factor": 4.0, "fast": 32.0, "original": 2048, "slow": 1.0}}}
-    att = {"conv": v["taps"], "dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv"], "scale": s["dim"] ** -0.5, "softcap": 50.0, "vdim": s["dim"]}
+           "rot": {"base": 10000.0, "dims": v["l_rot"], "scaling": {"factor": 8.0, "fast": 24.0, "original": 4096, "slow": 2.0}}}
+    att = {"conv": v["taps"], "dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv"], "scale": s["dim"] ** -0.5, "softcap": 30.0, "vdim": s["dim"]}
     mlp = {"ff": s["ff"], "kind": "dense"}
     layers, first = [], {}
     for i, c in enumerate(v["layers"]):
@@ -41,7 +41,7 @@ def vivazen_config(s, v):
             e["weights_of"] = first["l"]
         first.setdefault(c, i)
         layers.append(e)
-    return {"architecture": "Vivazen", "layers": layers, "norm": {"eps": 1e-5, "groups": 4}, "postln_alpha": 3.0, "vocab": s["vocab"], "width": s["width"]}
+    return {"architecture": "Vivazen", "layers": layers, "norm": {"eps": 1e-6, "groups": 8}, "postln_alpha": 2.0, "vocab": s["vocab"], "width": s["width"]}
 
 
 def vivazen_shapes(cfg):

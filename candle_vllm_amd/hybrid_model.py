@@ -5,6 +5,7 @@ config.json (`architecture`, `layers`, `norm`, `vocab`, `width`, ...) becomes th
 host layer's slots.  No CPU fallback; torch only holds device buffers."""
 import ctypes
 import json
+import math
 import os
 import struct
 
@@ -187,6 +188,8 @@ class VivazenSpec:
         if sc:
             rs.type, rs.factor, rs.original_max_position_embeddings = ROPE_YARN, float(sc["factor"]), float(sc["original"])
             rs.beta_fast, rs.beta_slow, rs.attn_factor = float(sc["fast"]), float(sc["slow"]), 1.0
+            if rs.factor <= 1.0:              # the table builder keeps amplitude 1 up to factor 1; this design's 0.1 ln(factor) + 1 holds for every factor
+                rs.attn_factor = 0.1 * math.log(rs.factor) + 1.0
         else:
             rs.type = ROPE_DEFAULT
         return rs

@@ -124,7 +124,8 @@ def _tables(lib, dims, n_pos, base, scaling):
     return cos, sin
 
 
-@pytest.mark.parametrize("dims,base,scaling", [(16, 50000.0, {"factor": 4.0, "fast": 32.0, "original": 2048, "slow": 1.0}),
+@pytest.mark.parametrize("dims,base,scaling", [(16, 20000.0, {"factor": 6.0, "fast": 16.0, "original": 1024, "slow": 1.5}),
+                                               (10, 300.0, {"factor": 0.5, "fast": 3.0, "original": 48, "slow": 0.25}),       # a factor below 1: amplitude below 1
                                                (8, 100.0, {"factor": 2.5, "fast": 4.0, "original": 64, "slow": 0.5}),
                                                (32, 1e6, {"factor": 16.0, "fast": 8.0, "original": 512, "slow": 2.0}),
                                                (2, 10.0, {"factor": 3.0, "fast": 32.0, "original": 32, "slow": 1.0}),
@@ -136,7 +137,8 @@ def test_yarn_tables(lib, dims, base, scaling):
     assert np.abs(cos - np.cos(ang) * amp).max() < 2e-7 * amp and np.abs(sin - np.sin(ang) * amp).max() < 2e-7 * amp
     if scaling:
         plain, _ = V.yarn_frequencies(base, dims, None)
-        assert amp > 1.0 and np.all(f <= plain + 1e-18) and np.all(f >= plain / scaling["factor"] - 1e-18)
+        lo, hi = sorted((1.0, 1.0 / scaling["factor"]))
+        assert (amp > 1.0) == (scaling["factor"] > 1.0) and np.all(f <= plain * hi + 1e-18) and np.all(f >= plain * lo - 1e-18)
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -375,11 +377,11 @@ def small_config(variant=0):
         cfg = {"architecture": "Vivazen", "layers": layers, "norm": {"eps": 1e-3, "groups": 1}, "postln_alpha": 1.0, "vocab": 33, "width": 40}
     if variant == 2:                # sizes that take the matrix-core attention in bf16 prompts: 64-wide latent rows, 32-wide heads
         lat2 = {"dim": 16, "heads": 4, "kv_rank": 48, "rot_dim": 16, "vdim": 24, "scale": 0.2, "mask": {"size": 70},
-                "rot": {"base": 5e4, "dims": 16, "scaling": {"factor": 4.0, "fast": 32.0, "original": 128, "slow": 1.0}}}
+                "rot": {"base": 2e4, "dims": 16, "scaling": {"factor": 5.0, "fast": 20.0, "original": 128, "slow": 2.0}}}
         att2 = {"conv": 3, "dim": 32, "heads": 4, "kv_heads": 2, "scale": 0.2, "softcap": 20.0, "vdim": 16}
         layers = [{"type": "latent_attention", "mixer": lat2, "mlp": mlp}, {"type": "attention", "mixer": att2, "mlp": mlp},
                   {"type": "latent_attention", "mixer": lat2, "mlp": mlp, "weights_of": 0}]
-        cfg = {"architecture": "Vivazen", "layers": layers, "norm": {"eps": 1e-5, "groups": 2}, "postln_alpha": 3.0, "vocab": 120, "width": 64}
+        cfg = {"architecture": "Vivazen", "layers": layers, "norm": {"eps": 1e-5, "groups": 2}, "postln_alpha": 1.5, "vocab": 120, "width": 64}
     return cfg
 
 
