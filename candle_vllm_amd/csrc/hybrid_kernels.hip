@@ -466,6 +466,7 @@ struct AttnArgs {
     int k_ld, v_ld;         // elements per page row (all key/value heads of a token; latent attention: one row serves as both)
     float softcap;          // > 0: score <- cap tanh(score / cap)
     int cross;              // blockIdx.z = the key/value head whose VALUES this block sums (scores still against the head's own keys)
+    int cpk;                // lanes that share a key row when it is read 16 bytes a lane (power of two >= d / elements per 16 bytes)
 };
 __device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 // 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
@@ -491,7 +492,7 @@ template <> struct Vec16<float> {
 // partial results are merged through LDS.  The sink enters the merge as a partial result with maximum sink, denominator 1 and no
 // value.  VEC (head sizes that are multiples of 16 bytes): rows are read 16 bytes at a time; for the value sum the wave's lanes
 // are (key, 16-byte chunk of the row) pairs -- 64 / cp2 keys per pass -- and the keys' partial sums are added by lane exchanges.
-// DQ > 0 (VEC, d = DQ): the query sits in registers, so a key's score costs its 16-byte loads and d FMAs and nothing else.
+// (DQ: unused, 0.)
 // NV > 1 (cross mode): the head's weights are applied to the values of NV key/value heads; the scores are computed once.
 template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bounds__(64 * NW) void window_attention_kernel(AttnArgs p) {
     constexpr int EPV = Vec16<TC>::N;
@@ -511,14 +512,17 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
     const TC* q = static_cast<const TC*>(p.q) + ((size_t)t * p.H + h) * p.d;
     for (int i = threadIdx.x; i < p.d; i += blockDim.x) qs[i] = ld<TC>(q, i);
     __syncthreads();
-    float qr[DQ > 0 ? DQ : 1];
-    if (DQ > 0) {
-#pragma unroll
-        for (int i = 0; i < DQ; ++i) qr[i] = qs[i];
-    }
     const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
     const int cp2 = p.cp2, chunk = lane & (cp2 - 1), ksub = lane / cp2, kpp = 64 / cp2;     // VEC only
     const bool chunk_ok = chunk * EPV < p.vd;
+    // VEC scores: lanes are (key, 16-byte chunk of its row) pairs too -- kq keys per pass, a pass reads kq whole rows (a lane per
+    // 16 bytes, neighbouring lanes neighbouring bytes) instead of 16 bytes of 64 different rows; the chunk of the query that a lane
+    // multiplies stays in its registers
+    const int cpk = p.cpk, qchunk = lane & (cpk - 1), qsub = lane / cpk, kq = 64 / cpk;
+    const bool qok = qchunk * EPV < p.d;
+    float qv[EPV];
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) qv[e] = (VEC && qok) ? qs[qchunk * EPV + e] : 0.f;
     float m = -INFINITY, l = 0.f, acc[NV][NACC];
 #pragma unroll
     for (int n = 0; n < NV; ++n)
@@ -526,30 +530,42 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
         for (int e = 0; e < NACC; ++e) acc[n][e] = 0.f;
     for (int j0 = lo + wave * 64; j0 <= pos; j0 += NW * 64) {
         const int j = j0 + lane;
+        const int cnt = min(64, pos - j0 + 1);
         float sc = -INFINITY;
         unsigned page_row = 0;
-        if (j <= pos) {
-            page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
+        if (j <= pos) page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
+        if (VEC) {
+            constexpr int SU = 8;                                         // passes whose loads are in flight together
+            float dot = 0.f;
+            const int qcol = g * p.d + (qok ? qchunk * EPV : 0);
+            for (int u0 = 0; u0 * kq < cnt; u0 += SU) {
+                float part[SU];
+#pragma unroll
+                for (int u = 0; u < SU; ++u) {
+                    const int jj = (u0 + u) * kq + qsub;
+                    const bool on = jj < cnt && qok;
+                    const size_t pr = (size_t)__shfl(page_row, jj & 63);
+                    float x[EPV];
+                    Vec16<TC>::load(static_cast<const TC*>(p.k_pages) + (on ? pr : (size_t)0) * p.k_ld + qcol, x);
+                    float a = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPV; ++e) a = fmaf(qv[e], x[e], a);
+                    part[u] = on ? a : 0.f;
+                }
+                for (int o = 1; o < cpk; o <<= 1)
+#pragma unroll
+                    for (int u = 0; u < SU; ++u) part[u] += __shfl_xor(part[u], o);
+#pragma unroll
+                for (int u = 0; u < SU; ++u) {                            // the lane that owns key (u0 + u) kq + i takes it from group i
+                    const float v = __shfl(part[u], (lane % kq) * cpk);
+                    if (lane / kq == u0 + u) dot = v;
+                }
+            }
+            if (j <= pos) sc = cap_score(dot * p.scale, p.softcap);
+        } else if (j <= pos) {
             const TC* kr = static_cast<const TC*>(p.k_pages) + (size_t)page_row * p.k_ld + g * p.d;
             float dot = 0.f;
-            if (VEC && DQ > 0) {
-#pragma unroll
-                for (int i = 0; i < DQ; i += EPV) {
-                    float x[EPV];
-                    Vec16<TC>::load(kr + i, x);
-#pragma unroll
-                    for (int e = 0; e < EPV; ++e) dot = fmaf(qr[i + e], x[e], dot);
-                }
-            } else if (VEC) {
-                for (int i = 0; i < p.d; i += EPV) {
-                    float x[EPV];
-                    Vec16<TC>::load(kr + i, x);
-#pragma unroll
-                    for (int e = 0; e < EPV; ++e) dot = fmaf(qs[i + e], x[e], dot);
-                }
-            } else {
-                for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
-            }
+            for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
             sc = cap_score(dot * p.scale, p.softcap);
         }
         const float mn = fmaxf(m, wave_max(sc));
@@ -561,21 +577,31 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
 #pragma unroll
             for (int e = 0; e < NACC; ++e) acc[n][e] *= corr;
         m = mn;
-        const int cnt = min(64, pos - j0 + 1);
         if (VEC) {
-            for (int k0 = 0; k0 < cnt; k0 += kpp) {
-                const int jj = k0 + ksub;
-                const float pv = __shfl(pj, jj & 63);
-                const size_t pr = (size_t)__shfl(page_row, jj & 63);
-                if (jj < cnt && chunk_ok) {
+            // PU passes of kpp keys at a time: the value rows of all of them are requested before the first is summed, so a chunk
+            // costs 64 / (kpp PU) memory round trips instead of 64 / kpp.  A pass beyond the chunk's end (or a lane whose 16-byte
+            // chunk lies beyond the row) reads a valid row with weight 0 and its values are replaced by zeros.
+            constexpr int PU = NV >= 2 ? 2 : 8;
+            const int vcol = chunk_ok ? chunk * EPV : 0;
+            for (int k0 = 0; k0 < cnt; k0 += kpp * PU) {
+                float pv[PU], x[PU][NV][EPV];
 #pragma unroll
-                    for (int n = 0; n < NV; ++n) {
-                        float x[EPV];
-                        Vec16<TC>::load(static_cast<const TC*>(p.v_pages) + pr * p.v_ld + (gv0 + n) * p.vd + chunk * EPV, x);
+                for (int u = 0; u < PU; ++u) {
+                    const int jj = k0 + u * kpp + ksub;
+                    const bool on = jj < cnt && chunk_ok;
+                    const float pjj = __shfl(pj, jj & 63);
+                    pv[u] = on ? pjj : 0.f;
+                    const size_t pr = (size_t)__shfl(page_row, jj & 63);
+                    const TC* vr = static_cast<const TC*>(p.v_pages) + (on ? pr : (size_t)0) * p.v_ld + gv0 * p.vd + vcol;
 #pragma unroll
-                        for (int e = 0; e < EPV; ++e) acc[n][e] = fmaf(pv, x[e], acc[n][e]);
-                    }
+                    for (int n = 0; n < NV; ++n) Vec16<TC>::load(vr + n * p.vd, x[u][n]);
                 }
+#pragma unroll
+                for (int u = 0; u < PU; ++u)
+#pragma unroll
+                    for (int n = 0; n < NV; ++n)
+#pragma unroll
+                        for (int e = 0; e < EPV; ++e) acc[n][e] = fmaf(pv[u], pv[u] != 0.f ? x[u][n][e] : 0.f, acc[n][e]);
             }
         } else {
             for (int jj = 0; jj < cnt; ++jj) {
@@ -1372,9 +1398,10 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
                k_ld, v_ld, softcap, cross};
     hipStream_t s_ = to_stream(stream);
     const int epv = f ? 4 : 8;
-    const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 &&
+    const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && dim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 &&
                      k_ld % epv == 0 && v_ld % epv == 0;
-    if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; }
+    p.cpk = 64;
+    if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; c = 1; while (c < dim / epv) c <<= 1; p.cpk = c; }
     else if (vdim > 512) return -1;
     // prompt-sized steps over bf16 pages: the matrix-core kernel (a tile of 16 tokens never spans two sequences)
     if (!f && T >= 64 && dim % 32 == 0 && dim <= 256 && vdim % 16 == 0 && vdim <= 256 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
@@ -1409,15 +1436,14 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
     }
     // few (token, head) pairs (decoding batches): eight waves share a window instead of four
     const bool wide = (int64_t)T * heads < 2048;
-    const int dq = !vec ? 0 : dim == 64 ? 64 : dim == 128 ? 128 : 0;
     // cross mode with 16-byte rows: 4 or 2 value heads per workgroup, the rest of the key/value heads along z
     int nv = (cross && vec) ? (kv_heads % 4 == 0 ? 4 : kv_heads % 2 == 0 ? 2 : 1) : 1;
     if ((size_t)8 * nv * vdim * sizeof(float) > 32768) nv = 1;          // the waves' partial sums must fit the workgroup's LDS
+    while (nv > 1 && (int64_t)T * heads * (nz / nv) < 512) nv >>= 1;    // decoding batches: rather more workgroups than shared scores
     const dim3 ggrid(T, heads, nz / nv);
 #define WA4(TC, NW, VEC, DQ, NV) window_attention_kernel<TC, NW, VEC, DQ, NV><<<ggrid, 64 * NW, (size_t)(((dim + 3) & ~3) + 2 * NW + NW * NV * vdim) * sizeof(float), s_>>>(p)
 #define WA3(TC, NW, VEC, DQ) do { if (nv == 4) WA4(TC, NW, VEC, DQ, 4); else if (nv == 2) WA4(TC, NW, VEC, DQ, 2); else WA4(TC, NW, VEC, DQ, 1); } while (0)
-#define WA2(TC, NW) do { if (!vec) WA4(TC, NW, false, 0, 1); else if (dq == 64) WA3(TC, NW, true, 64); else if (dq == 128) WA3(TC, NW, true, 128); \
-                         else WA3(TC, NW, true, 0); } while (0)
+#define WA2(TC, NW) do { if (!vec) WA4(TC, NW, false, 0, 1); else WA3(TC, NW, true, 0); } while (0)
 #define WA(TC) do { if (wide) WA2(TC, 8); else WA2(TC, 4); } while (0)
     if (f) WA(float); else WA(uint16_t);
 #undef WA
