@@ -658,13 +658,18 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
 //   (lane (m16, kg) = 16 bytes of key m16 of a 16-key tile); the accumulator holds queries 4 kg + v against key m16.
 //   Mask, scale and the online softmax run on that layout in f32 (row maxima / sums: exchanges among the 16 lanes of a kg group).
 //   P V: the probabilities go through LDS into A-fragment order as TWO bf16 planes (p = hi + lo, so the weights keep about 16 bits
-//   of mantissa), the 64 value rows are transposed through LDS ([column][key]) so that a B fragment is one 16-byte read.
+//   of mantissa), the 64 value rows go through LDS to become B fragments (8 keys of one column per lane).
 // The sink is applied at the end: denominator += exp(sink - max).
 // NV > 1 (cross mode): the block applies its head's weights to the values of NV key/value heads one after the other -- Q K^T, the
 // softmax and the probability planes are made once per chunk, the transposed value tile in LDS is refilled per value head.
-template <int DK, int VT, int NV> __global__ __launch_bounds__(64) void window_attention_mfma_kernel(AttnArgs p) {
+template <int DK, int VT, int NV> __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(NV == 2 ? 2 : 1)))
+void window_attention_mfma_kernel(AttnArgs p) {
     constexpr int RS = 72;                                           // bf16 per LDS row: 64 keys + 8 of padding (144 bytes)
-    __shared__ __align__(16) uint16_t Ph[16 * RS], Pl[16 * RS], Vt[VT * 16 * RS];
+    // NV > 1: the value rows lie in LDS as rows (VRS bf16 each: 8 rows on are 16 banks on) and a B fragment gathers its 8 keys of one
+    // column with 2-byte reads; NV == 1: they are transposed by the store ([column][key]) and a B fragment is one 16-byte read
+    constexpr bool ROWS = NV > 1;
+    constexpr int VRS = VT * 16 + 4;
+    __shared__ __align__(16) uint16_t Ph[16 * RS], Pl[16 * RS], Vt[ROWS ? 64 * VRS : VT * 16 * RS];
     const int lane = threadIdx.x, m16 = lane & 15, kg = lane >> 4;
     int b = blockIdx.x, s = 0, n_new = 0;
     for (; s < p.n_seqs; ++s) {
@@ -712,6 +717,14 @@ template <int DK, int VT, int NV> __global__ __launch_bounds__(64) void window_a
         // even lane keeps the even column of both keys and the odd lane the odd column, so every lane writes ONE 4-byte word (two
         // keys of one column) instead of two 2-byte halves
         auto stage_values = [&]() {
+            if (ROWS) {
+#pragma unroll
+                for (int c8 = 0; c8 < VT * 2; ++c8) {
+                    *reinterpret_cast<uint2*>(&Vt[lane * VRS + c8 * 8]) = uint2{vreg[c8].x, vreg[c8].y};
+                    *reinterpret_cast<uint2*>(&Vt[lane * VRS + c8 * 8 + 4]) = uint2{vreg[c8].z, vreg[c8].w};
+                }
+                return;
+            }
             const int col_odd = lane & 1, key_even = lane & ~1;
 #pragma unroll
             for (int c8 = 0; c8 < VT * 2; ++c8) {
@@ -723,6 +736,16 @@ template <int DK, int VT, int NV> __global__ __launch_bounds__(64) void window_a
                     *reinterpret_cast<uint32_t*>(&Vt[(c8 * 8 + 2 * e + col_odd) * RS + key_even]) = pair;
                 }
             }
+        };
+        auto value_fragment = [&](int k2, int c) {
+            if (!ROWS) return *reinterpret_cast<const uint4*>(&Vt[(c * 16 + m16) * RS + k2 * 32 + 8 * kg]);
+            const uint16_t* col = &Vt[(k2 * 32 + 8 * kg) * VRS + c * 16 + m16];
+            uint4 f;
+            f.x = (uint32_t)col[0] | ((uint32_t)col[VRS] << 16);
+            f.y = (uint32_t)col[2 * VRS] | ((uint32_t)col[3 * VRS] << 16);
+            f.z = (uint32_t)col[4 * VRS] | ((uint32_t)col[5 * VRS] << 16);
+            f.w = (uint32_t)col[6 * VRS] | ((uint32_t)col[7 * VRS] << 16);
+            return f;
         };
         fetch_values(0);
         f32x4_t sacc[4];
@@ -797,7 +820,7 @@ template <int DK, int VT, int NV> __global__ __launch_bounds__(64) void window_a
             for (int k2 = 0; k2 < 2; ++k2)
 #pragma unroll
                 for (int c = 0; c < VT; ++c) {
-                    const uint4 vf = *reinterpret_cast<const uint4*>(&Vt[(c * 16 + m16) * RS + k2 * 32 + 8 * kg]);
+                    const uint4 vf = value_fragment(k2, c);
                     acc[n][c] = mfma_bf16(ah[k2], vf, acc[n][c]);
                     acc[n][c] = mfma_bf16(al[k2], vf, acc[n][c]);
                 }
@@ -1407,13 +1430,12 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
     if (!f && T >= 64 && dim % 32 == 0 && dim <= 256 && vdim % 16 == 0 && vdim <= 256 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
         (uintptr_t)v_pages % 16 == 0 && k_ld % 8 == 0 && v_ld % 8 == 0 && g_attn_mfma) {
         const int dk = dim / 32, vt = vdim / 16;
-        // cross mode: 4 or 2 value heads per block where the head sizes have such a build (dim <= 128, vdim <= 128), the rest of
-        // the key/value heads along z
-        const int nv = (cross && dk <= 4 && vt <= 8) ? (kv_heads % 4 == 0 ? 4 : kv_heads % 2 == 0 ? 2 : 1) : 1;
+        // cross mode: 2 value heads per block where the head sizes have such a build (dim <= 128, vdim <= 128), the rest of the
+        // key/value heads along z (4 per block: one wave per SIMD, measured 1.4 x slower)
+        const int nv = (cross && dk <= 4 && vt <= 8) ? (kv_heads % 2 == 0 ? 2 : 1) : 1;
         const dim3 mgrid((T + 15) / 16 + num_seqs, heads, nz / nv);
 #define WM1(DK, VT) window_attention_mfma_kernel<DK, VT, 1><<<mgrid, 64, 0, s_>>>(p)
-#define WMN(DK, VT) do { if (nv == 4) window_attention_mfma_kernel<DK, VT, 4><<<mgrid, 64, 0, s_>>>(p); \
-                         else if (nv == 2) window_attention_mfma_kernel<DK, VT, 2><<<mgrid, 64, 0, s_>>>(p); else WM1(DK, VT); } while (0)
+#define WMN(DK, VT) do { if (nv == 2) window_attention_mfma_kernel<DK, VT, 2><<<mgrid, 64, 0, s_>>>(p); else WM1(DK, VT); } while (0)
 #define WMV(DK, WM) do { switch (vt) { case 1: WM(DK, 1); break; case 2: WM(DK, 2); break; case 3: WM(DK, 3); break; case 4: WM(DK, 4); break; \
                                         case 5: WM(DK, 5); break; case 6: WM(DK, 6); break; case 7: WM(DK, 7); break; case 8: WM(DK, 8); break; \
                                         default: ok_shape = false; } } while (0)
