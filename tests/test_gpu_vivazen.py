@@ -619,3 +619,86 @@ def test_greedy_generation_through_scheduler(lib, chunk):
     for r, w in zip(reqs, want):
         assert r.tokens == w, (r.id, r.tokens, w)
     assert sched.block_engine.state_free_slots() == 4
+
+
+# ------------------------------------------------------------------------------------------------------------ random configurations
+def random_config(rng):
+    """sizes, head counts, layer order, windows and constants drawn at random (sizes of 8 .. 192 that are not all multiples of 16 or 32,
+    one to eight heads, two to five taps, one to eight norm groups, layers that borrow an earlier layer's weights, layers without a
+    feed-forward, rotation with and without scaling)"""
+    width = int(rng.choice([96, 128, 192, 256, 320, 384]))
+    groups = int(rng.choice([g for g in (1, 2, 3, 4, 6, 8) if width % g == 0]))
+
+    def lat():
+        d, r = int(rng.choice([16, 24, 32, 48, 64, 96, 128])), int(rng.choice([4, 8, 16, 32, 64]))
+        m = {"dim": d, "heads": int(rng.choice([1, 2, 3, 4, 6, 8])), "kv_rank": int(rng.choice([16, 24, 32, 48, 64, 96, 128, 192])), "rot_dim": r,
+             "vdim": int(rng.choice([8, 16, 24, 32, 48, 64, 96])), "scale": float((d + r) ** -0.5 * rng.uniform(0.7, 1.5)),
+             "mask": {"size": int(rng.integers(5, 200))}, "rot": {"base": float(rng.choice([1e3, 1e4, 5e5, 123456.0])), "dims": r}}
+        if rng.random() < 0.8:
+            m["rot"]["scaling"] = {"factor": float(rng.choice([2.0, 3.5, 8.0, 16.0, 40.0])), "fast": float(rng.choice([8.0, 16.0, 32.0, 64.0])),
+                                   "original": int(rng.choice([64, 256, 1024, 4096])), "slow": float(rng.choice([0.5, 1.0, 2.0]))}
+        return m
+
+    def att():
+        G, d = int(rng.choice([1, 2, 3, 4])), int(rng.choice([16, 32, 40, 64, 80, 128]))
+        return {"conv": int(rng.integers(2, 6)), "dim": d, "heads": G * int(rng.choice([1, 2, 3, 4])), "kv_heads": G,
+                "scale": float(d ** -0.5 * rng.uniform(0.7, 1.5)), "softcap": float(rng.choice([5.0, 20.0, 50.0, 100.0])),
+                "vdim": int(rng.choice([8, 16, 24, 48, 64, 80, 128]))}
+    kinds = {"latent_attention": [lat() for _ in range(2)], "attention": [att() for _ in range(2)]}
+    layers = []
+    for _ in range(int(rng.integers(3, 9))):
+        owners = [j for j, l in enumerate(layers) if "weights_of" not in l]
+        if owners and rng.random() < 0.3:
+            j = int(rng.choice(owners))
+            layers.append(dict(layers[j], weights_of=j))
+            continue
+        t = str(rng.choice(["latent_attention", "attention"]))
+        layers.append({"type": t, "mixer": kinds[t][int(rng.integers(0, 2))],
+                       "mlp": {"ff": int(rng.choice([64, 160, 384, 512])), "kind": "dense"} if rng.random() < 0.85 else None})
+    return {"architecture": "Vivazen", "layers": layers, "norm": {"eps": float(rng.choice([1e-5, 1e-6])), "groups": groups},
+            "postln_alpha": float(rng.choice([2.0, 3.0, 4.0])), "vocab": int(rng.integers(50, 600)), "width": width}
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seed", [2, 3, 11, 21])
+def test_random_configurations_whole_and_mixed_schedules(lib, seed):
+    """three unequal requests of a random configuration: each alone in one step, then together in a random schedule of portions (2, 3,
+    17, 64, 65, 100 tokens; a request may sit a step out) that ends token by token -- on 64-token pages, in f32 and bf16"""
+    _gpu()
+    from candle_vllm_amd.step_engine import StepEngine
+    rng = np.random.default_rng(seed)
+    cfg = random_config(rng)
+    W = V.random_vivazen(rng, cfg)
+    lens = [int(rng.integers(150, 420)), int(rng.integers(1, 40)), int(rng.integers(60, 130))]
+    toks = [rng.integers(0, cfg["vocab"], n).tolist() for n in lens]
+    want = [V.VivazenOracle(cfg, W).feed(t)[0] for t in toks]
+    from candle_vllm_amd.hybrid_model import HybridModel, VivazenSpec
+    for dtype in ("float32", "bfloat16"):
+        m = HybridModel(VivazenSpec(cfg, {k: v.shape for k, v in W.items()}), dtype=dtype, block_size=64, state_slots=4)
+        m.load_state_dict_f32(W)
+        eng = StepEngine(m, 64 * 12)
+        for i, t in enumerate(toks):
+            eng.feed("w", t)
+            assert row_err(eng.step(["w"], [list(range(len(t)))]).cpu().numpy(), want[i]) < TOL[dtype], (dtype, "whole", i)
+            eng.finish("w")
+        at, got = [0, 0, 0], [[], [], []]
+        while any(a < n for a, n in zip(at, lens)):
+            ids, w, take = [], [], []
+            for i in range(3):
+                if at[i] >= lens[i] or rng.random() < 0.2:
+                    continue
+                left = lens[i] - at[i]
+                c = 1 if left <= 20 else int(min(left - 20, rng.choice([2, 3, 17, 64, 65, 100])))
+                eng.feed("r%d" % i, toks[i][at[i]:at[i] + c])
+                ids.append("r%d" % i); w.append(list(range(c))); take.append((i, c))
+                at[i] += c
+            if not ids:
+                continue
+            out, lo = eng.step(ids, w).cpu().numpy(), 0
+            for i, c in take:
+                got[i].append(out[lo:lo + c]); lo += c
+                if at[i] == lens[i]:
+                    eng.finish("r%d" % i)
+        for i in range(3):
+            assert row_err(np.concatenate(got[i]), want[i]) < TOL[dtype], (dtype, "schedule", i)
+        assert eng.free_pages() == eng.num_blocks and eng.be.state_free_slots() == 4
