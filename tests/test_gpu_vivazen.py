@@ -660,7 +660,7 @@ def random_config(rng):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("seed", [2, 3, 11, 21])
+@pytest.mark.parametrize("seed", [2, 11, 21])
 def test_random_configurations_whole_and_mixed_schedules(lib, seed):
     """three unequal requests of a random configuration: each alone in one step, then together in a random schedule of portions (2, 3,
     17, 64, 65, 100 tokens; a request may sit a step out) that ends token by token -- on 64-token pages, in f32 and bf16"""
